@@ -12,6 +12,9 @@
 //                      vectors per head (q also times D^-1/2), beta = sigmoid(b),
 //                      g = exp(-exp(A_log) softplus(a + dt_bias))
 //   conv_keep          the step's last taps-1 inputs into the request's state
+//   causal_conv        the short causal convolution alone, for any mixer: per channel, with an optional bias and
+//                      silu, from the same kind of kept inputs; the result in 32-bit and, if wanted, once more
+//                      in the type of the product that reads it next
 //   gated_delta_scan   the recurrence; o in 32-bit
 //
 // With old state S, ks = S^T k and qs = S^T q (both from the old S, so their sums run side by side):
@@ -125,6 +128,33 @@ __global__ void conv_keep_kernel(const float* __restrict__ proj, int64_t stride,
     fresh[i] = x;
   }
   for (int i = 0; i < taps - 1; ++i) kept[(int64_t)i * channels + c] = fresh[i];
+}
+
+// A thread a (row, channel). x [rows][stride] holds the inputs of `channels` channels from column 0.
+template <typename T>
+__global__ void causal_conv_kernel(const float* __restrict__ x, int64_t stride, const float* __restrict__ conv_w,
+                                   const float* __restrict__ bias, const float* kept_base, int64_t state_stride,
+                                   const int* __restrict__ q_start, int entries, const int* __restrict__ positions,
+                                   const int* __restrict__ state_slots, float* __restrict__ out, int64_t out_stride,
+                                   T* __restrict__ rounded, int64_t rounded_stride, int channels, int taps, int act) {
+  const int row = blockIdx.x;
+  const int c = blockIdx.y * blockDim.x + threadIdx.x;
+  if (c >= channels) return;
+  const int e = gd_entry_of_row(q_start, entries, row);
+  const int first = q_start[e], pos = positions[row];
+  const float* kept = kept_base + (int64_t)state_slots[e] * state_stride;
+  float acc = bias != nullptr ? bias[c] : 0.f;
+  for (int j = taps - 1; j >= 0; --j) {                          // oldest input first
+    float in = 0.f;
+    if (pos - j >= 0) {
+      const int src = row - j;
+      in = src >= first ? x[(int64_t)src * stride + c] : kept[(int64_t)(taps - 1 - (first - src)) * channels + c];
+    }
+    acc = fmaf(conv_w[(int64_t)c * taps + (taps - 1 - j)], in, acc);
+  }
+  if (act == 1) acc = acc / (1.f + expf(-acc));
+  out[(int64_t)row * out_stride + c] = acc;
+  if (rounded != nullptr) rounded[(int64_t)row * rounded_stride + c] = from_f32<T>(acc);
 }
 
 struct GdArgs {
@@ -299,6 +329,35 @@ int dli_conv_prepare(const float* proj, int64_t stride, int b_off, int a_off, co
     const dim3 grid(entries, (unsigned)((channels + 255) / 256));
     conv_keep_kernel<<<grid, 256, 0, stream>>>(proj, stride, state + kept_offset, state_stride, q_start, positions,
                                                state_slots, (int)channels, taps);
+  }
+  return dli_launch_status();
+}
+
+// act: 0 none, 1 silu. rounded (may be nullptr): the result once more, bf16 if rounded_is_bf16 else float.
+int dli_causal_conv(const float* x, int64_t stride, const float* conv_w, const float* bias, float* state,
+                    int64_t state_stride, int64_t kept_offset, const int* q_start, const int* positions,
+                    const int* state_slots, float* out, int64_t out_stride, void* rounded, int64_t rounded_stride,
+                    int rounded_is_bf16, int entries, int rows, int channels, int taps, int act, hipStream_t stream) {
+  if (rows <= 0 || entries <= 0) return DLI_OK;
+  if (channels <= 0 || taps < 1 || taps > GD_MAX_TAPS || stride < channels || out_stride < channels ||
+      (rounded != nullptr && rounded_stride < channels) || act < 0 || act > 1 ||
+      state_stride < kept_offset + (int64_t)(taps - 1) * channels)
+    return DLI_ERR_ARGUMENT;
+  const dim3 grid(rows, (channels + 255) / 256);
+  if (grid.y > 65535) return DLI_ERR_ARGUMENT;
+  if (rounded_is_bf16)
+    causal_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>(x, stride, conv_w, bias, state + kept_offset, state_stride, q_start,
+                                                         entries, positions, state_slots, out, out_stride, (bf16_t*)rounded,
+                                                         rounded_stride, channels, taps, act);
+  else
+    causal_conv_kernel<float><<<grid, 256, 0, stream>>>(x, stride, conv_w, bias, state + kept_offset, state_stride, q_start,
+                                                        entries, positions, state_slots, out, out_stride, (float*)rounded,
+                                                        rounded_stride, channels, taps, act);
+  if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
+  if (taps > 1) {
+    const dim3 keep(entries, (channels + 255) / 256);
+    conv_keep_kernel<<<keep, 256, 0, stream>>>(x, stride, state + kept_offset, state_stride, q_start, positions,
+                                               state_slots, channels, taps);
   }
   return dli_launch_status();
 }

@@ -33,6 +33,7 @@
 
 #define RULE_DELTA 0
 #define RULE_BONUS 1
+#define GATE_NONE 2   // head_norm_gate alone: the per-head norm without a gate
 
 struct ScanArgs {
   const float* r; const float* k; const float* v;   // [rows][heads * D], each with its row stride
@@ -248,8 +249,11 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
     for (int c = lane; c < dim; c += DLI_WAVE) ss += oh[c] * oh[c];
     const float r = 1.f / sqrtf(wave_sum(ss) / (float)dim + eps);
     for (int c = lane; c < dim; c += DLI_WAVE) {
-      const float g = g_pre[row * g_stride + (int64_t)h * dim + c];
-      const float gate = RULE == RULE_DELTA ? 1.f / (1.f + expf(-g)) : g / (1.f + expf(-g));
+      float gate = 1.f;                                   // RULE 2: no gate (g_pre is not read)
+      if (RULE != GATE_NONE) {
+        const float g = g_pre[row * g_stride + (int64_t)h * dim + c];
+        gate = RULE == RULE_DELTA ? 1.f / (1.f + expf(-g)) : g / (1.f + expf(-g));
+      }
       out[row * out_stride + (int64_t)h * dim + c] = from_f32<T>(oh[c] * r * norm_w[(int64_t)h * dim + c] * gate);
     }
   }
@@ -322,15 +326,18 @@ extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float*
 // norm_w holds heads * dim values (a weight that the heads share is repeated by the caller).
 extern "C" int dli_head_norm_gate(const float* o, int64_t o_stride, const float* g_pre, int64_t g_stride,
                                   const float* norm_w, float eps, void* out, int64_t out_stride, int rows, int heads,
-                                  int dim, int gate_silu, int out_is_bf16, hipStream_t stream) {
+                                  int dim, int gate, int out_is_bf16, hipStream_t stream) {
+  // gate: 0 sigmoid(g_pre), 1 silu(g_pre), 2 none
   if (rows <= 0) return DLI_OK;
   const int64_t width = (int64_t)heads * dim;
-  if (heads <= 0 || dim <= 0 || o_stride < width || g_stride < width || out_stride < width) return DLI_ERR_ARGUMENT;
+  if (heads <= 0 || dim <= 0 || o_stride < width || out_stride < width || gate < 0 || gate > 2 ||
+      (gate != GATE_NONE && (g_pre == nullptr || g_stride < width)))
+    return DLI_ERR_ARGUMENT;
   const dim3 grid(rows, (heads + 3) / 4);
   if (grid.y > 65535) return DLI_ERR_ARGUMENT;
 #define HNG(T, RULE) head_norm_gate_kernel<T, RULE><<<grid, 256, 0, stream>>>(o, o_stride, g_pre, g_stride, norm_w, eps, (T*)out, out_stride, heads, dim)
-  if (out_is_bf16) { if (gate_silu) HNG(bf16_t, RULE_BONUS); else HNG(bf16_t, RULE_DELTA); }
-  else { if (gate_silu) HNG(float, RULE_BONUS); else HNG(float, RULE_DELTA); }
+  if (out_is_bf16) { if (gate == GATE_NONE) HNG(bf16_t, GATE_NONE); else if (gate) HNG(bf16_t, RULE_BONUS); else HNG(bf16_t, RULE_DELTA); }
+  else { if (gate == GATE_NONE) HNG(float, GATE_NONE); else if (gate) HNG(float, RULE_BONUS); else HNG(float, RULE_DELTA); }
 #undef HNG
   return dli_launch_status();
 }

@@ -4,7 +4,8 @@
 //
 //   poly_norm        out(T) = a N(z) + b N(z^2) + c N(z^3) + e, powers element by element, N(x) = x / sqrt(mean(x^2) + eps)
 //                    over the row; z is the 32-bit result of the product before it
-//   clamped_glu      y = g sigmoid(alpha g) (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit)
+//   clamped_glu      y = g sigmoid(alpha g) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit); an infinite
+//                    limit, alpha 1 and shift 0 give the plain silu(gate) * up
 //   router_choose    softmax over all router outputs; choice = score + correction; only the `keep` groups of
 //                    neighbours with the largest best choice stay; the `top` largest choices; weights = the chosen
 //                    scores (without correction) / (their sum + 1e-20) * scale
@@ -48,18 +49,18 @@ __global__ void poly_norm_kernel_f32in(const float* __restrict__ z, int64_t z_st
   }
 }
 
-__device__ __forceinline__ float clamped_glu(float gate, float up, float limit, float alpha) {
+__device__ __forceinline__ float clamped_glu(float gate, float up, float limit, float alpha, float up_shift) {
   const float g = fminf(gate, limit), u = fminf(fmaxf(up, -limit), limit);
-  return g / (1.f + expf(-alpha * g)) * (u + 1.f);
+  return g / (1.f + expf(-alpha * g)) * (u + up_shift);
 }
 
 template <typename T>
 __global__ void clamped_glu_kernel(const T* __restrict__ gate_up, int64_t stride, T* __restrict__ out, int ff, float limit,
-                                   float alpha) {
+                                   float alpha, float up_shift) {
   const int64_t row = blockIdx.x;
   const int i = blockIdx.y * blockDim.x + threadIdx.x;
   if (i < ff)
-    out[row * ff + i] = from_f32<T>(clamped_glu(to_f32(gate_up[row * stride + i]), to_f32(gate_up[row * stride + ff + i]), limit, alpha));
+    out[row * ff + i] = from_f32<T>(clamped_glu(to_f32(gate_up[row * stride + i]), to_f32(gate_up[row * stride + ff + i]), limit, alpha, up_shift));
 }
 
 // The better of two (value, index) pairs: the larger value, the lower index on a tie.
@@ -74,6 +75,7 @@ __device__ __forceinline__ void wave_argmax(float& v, int& i) {
 
 // A wave a token. logits [rows][stride]: the first `total` columns are the router's outputs.
 __global__ __launch_bounds__(64) void router_choose_kernel(const float* __restrict__ logits, int64_t stride,
+                                                           const float* __restrict__ bias,
                                                            const float* __restrict__ correction, int total, int count,
                                                            int keep, int top, float scale, int* __restrict__ ids,
                                                            float* __restrict__ weights) {
@@ -83,11 +85,11 @@ __global__ __launch_bounds__(64) void router_choose_kernel(const float* __restri
   const int lane = threadIdx.x;
   const float* z = logits + row * stride;
   float m = -INFINITY;
-  for (int i = lane; i < total; i += DLI_WAVE) m = fmaxf(m, z[i]);
+  for (int i = lane; i < total; i += DLI_WAVE) m = fmaxf(m, z[i] + (bias != nullptr ? bias[i] : 0.f));
   m = wave_max(m);
   float sum = 0.f;
   for (int i = lane; i < total; i += DLI_WAVE) {
-    const float e = expf(z[i] - m);
+    const float e = expf(z[i] + (bias != nullptr ? bias[i] : 0.f) - m);
     s[i] = e;
     sum += e;
   }
@@ -200,7 +202,7 @@ struct ExpertArgs {
 template <typename T>
 __global__ __launch_bounds__(256) void expert_up_kernel(ExpertArgs p, const T* __restrict__ h, int64_t h_stride,
                                                         const T* __restrict__ w_gate, const T* __restrict__ w_up,
-                                                        T* __restrict__ y, float limit, float alpha) {
+                                                        T* __restrict__ y, float limit, float alpha, float up_shift) {
   const int tile = blockIdx.x;
   if (tile >= p.tile_count[0]) return;
   __shared__ float as[EX_BK][EX_BM + 1], gs[EX_BK][EX_BN + 4], us[EX_BK][EX_BN + 4];
@@ -246,7 +248,7 @@ __global__ __launch_bounds__(256) void expert_up_kernel(ExpertArgs p, const T* _
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int c = n0 + tx * 4 + j;
-      if (c < p.ff) y[(int64_t)r * p.ff + c] = from_f32<T>(clamped_glu(accg[i][j], accu[i][j], limit, alpha));
+      if (c < p.ff) y[(int64_t)r * p.ff + c] = from_f32<T>(clamped_glu(accg[i][j], accu[i][j], limit, alpha, up_shift));
     }
   }
 }
@@ -318,7 +320,7 @@ __device__ __forceinline__ exm_bf16x8 exm_load(const bf16_t* p) { return *reinte
 __global__ __launch_bounds__(256) void expert_up_mfma_kernel(ExpertArgs p, const bf16_t* __restrict__ h, int64_t h_stride,
                                                              const bf16_t* __restrict__ w_gate,
                                                              const bf16_t* __restrict__ w_up, bf16_t* __restrict__ y,
-                                                             float limit, float alpha) {
+                                                             float limit, float alpha, float up_shift) {
   const int tile = blockIdx.x;
   if (tile >= p.tile_count[0]) return;
   const int e = p.tile_expert[tile], r0 = p.tile_row0[tile], rend = p.offsets[e + 1];
@@ -378,7 +380,7 @@ __global__ __launch_bounds__(256) void expert_up_mfma_kernel(ExpertArgs p, const
       const int n0 = nw + nb * 16 + (lane / 16) * 4;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (n0 + i < p.ff) y[(int64_t)r * p.ff + n0 + i] = (bf16_t)clamped_glu(accg[nb][mb][i], accu[nb][mb][i], limit, alpha);
+        if (n0 + i < p.ff) y[(int64_t)r * p.ff + n0 + i] = (bf16_t)clamped_glu(accg[nb][mb][i], accu[nb][mb][i], limit, alpha, up_shift);
     }
   }
 }
@@ -472,23 +474,23 @@ int dli_poly_norm(const float* z, int64_t z_stride, const float* coef, void* out
   return dli_launch_status();
 }
 
-int dli_clamped_glu(const void* gate_up, int64_t stride, void* out, int rows, int ff, float limit, float alpha, int is_bf16,
+int dli_clamped_glu(const void* gate_up, int64_t stride, void* out, int rows, int ff, float limit, float alpha, float up_shift, int is_bf16,
                     hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (ff <= 0 || stride < 2 * (int64_t)ff) return DLI_ERR_ARGUMENT;
   const dim3 grid(rows, (ff + 255) / 256);
-  if (is_bf16) clamped_glu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, stride, (bf16_t*)out, ff, limit, alpha);
-  else clamped_glu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, stride, (float*)out, ff, limit, alpha);
+  if (is_bf16) clamped_glu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, stride, (bf16_t*)out, ff, limit, alpha, up_shift);
+  else clamped_glu_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, stride, (float*)out, ff, limit, alpha, up_shift);
   return dli_launch_status();
 }
 
-int dli_router_choose(const float* logits, int64_t stride, const float* correction, int rows, int total, int count, int keep,
+int dli_router_choose(const float* logits, int64_t stride, const float* bias, const float* correction, int rows, int total, int count, int keep,
                       int top, float scale, int* ids, float* weights, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   if (total <= 0 || total > 4096 || stride < total || top < 1 || top > 64 || top > total || count < 1 || total % count ||
       keep < 1 || keep > count || (int64_t)keep * (total / count) < top)
     return DLI_ERR_ARGUMENT;
-  router_choose_kernel<<<rows, 64, (2 * total + count) * sizeof(float), stream>>>(logits, stride, correction, total, count, keep,
+  router_choose_kernel<<<rows, 64, (2 * total + count) * sizeof(float), stream>>>(logits, stride, bias, correction, total, count, keep,
                                                                                   top, scale, ids, weights);
   return dli_launch_status();
 }
@@ -503,7 +505,7 @@ int dli_expert_tile_rows(int width, int ff, int is_bf16) { return expert_mfma(wi
 int dli_expert_products(const int* ids, const void* h, int64_t h_stride, const void* w_gate, const void* w_up,
                         const void* w_down, int* offsets, int* order, int* tile_expert, int* tile_row0, int* tile_count,
                         int max_tiles, void* y, float* z, int rows, int top, int experts, int width, int ff, float limit,
-                        float alpha, int is_bf16, hipStream_t stream) {
+                        float alpha, float up_shift, int is_bf16, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
   const int64_t slots = (int64_t)rows * top;
   if (top < 1 || experts < 1 || experts > 4096 || width <= 0 || ff <= 0 || h_stride < width || slots > (1 << 30) ||
@@ -523,15 +525,15 @@ int dli_expert_products(const int* ids, const void* h, int64_t h_stride, const v
   const dim3 up_grid(max_tiles, (ff + bn - 1) / bn), down_grid(max_tiles, (width + bn - 1) / bn);
   if (mfma) {
     expert_up_mfma_kernel<<<up_grid, 256, 0, stream>>>(p, (const bf16_t*)h, h_stride, (const bf16_t*)w_gate,
-                                                       (const bf16_t*)w_up, (bf16_t*)y, limit, alpha);
+                                                       (const bf16_t*)w_up, (bf16_t*)y, limit, alpha, up_shift);
     expert_down_mfma_kernel<<<down_grid, 256, 0, stream>>>(p, (const bf16_t*)y, (const bf16_t*)w_down, z);
   } else if (is_bf16) {
     expert_up_kernel<bf16_t><<<up_grid, 256, 0, stream>>>(p, (const bf16_t*)h, h_stride, (const bf16_t*)w_gate,
-                                                          (const bf16_t*)w_up, (bf16_t*)y, limit, alpha);
+                                                          (const bf16_t*)w_up, (bf16_t*)y, limit, alpha, up_shift);
     expert_down_kernel<bf16_t><<<down_grid, 256, 0, stream>>>(p, (const bf16_t*)y, (const bf16_t*)w_down, z);
   } else {
     expert_up_kernel<float><<<up_grid, 256, 0, stream>>>(p, (const float*)h, h_stride, (const float*)w_gate,
-                                                         (const float*)w_up, (float*)y, limit, alpha);
+                                                         (const float*)w_up, (float*)y, limit, alpha, up_shift);
     expert_down_kernel<float><<<down_grid, 256, 0, stream>>>(p, (const float*)y, (const float*)w_down, z);
   }
   return dli_launch_status();

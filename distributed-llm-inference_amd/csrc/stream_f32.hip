@@ -8,6 +8,8 @@
 //   norm_into_stream   x += w * y / sqrt(mean(y^2) + eps)   (a norm on a sublayer's output); like the embedding
 //                      it can leave the new stream once more in bf16, for the product that reads it next
 //   rms_norm_from_f32  out(T) = w * x / sqrt(mean(x^2) + eps)
+//   post_norm_stream   x <- w * s / sqrt(mean(s^2) + eps) with s = alpha x + r y, r = sigmoid(g + b) element by element
+//                      or 1 (a norm after the residual sum, the summand under a gate of its own)
 //   softcap            y = cap * tanh(y / cap)
 //   token_shift        S mixes of each row with the row before it, x + (prev - x) * mu_s; the row
 //                      before a step's first row comes from the request's state, which then
@@ -79,6 +81,31 @@ __global__ void rms_norm_from_f32_kernel(const float* __restrict__ x, const floa
   for (int i = threadIdx.x; i < width; i += blockDim.x) out[row * width + i] = from_f32<T>(weight[i] * (xr[i] * r));
 }
 
+// A workgroup a row. Each thread reads back only what it wrote itself.
+template <typename Y, typename R>
+__global__ void post_norm_stream_kernel(const Y* __restrict__ y, int64_t y_stride, const float* __restrict__ g,
+                                        int64_t g_stride, const float* __restrict__ g_bias,
+                                        const float* __restrict__ weight, float* __restrict__ x, R* __restrict__ rounded,
+                                        int width, float alpha, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    float t = to_f32(y[row * y_stride + i]);
+    if (g != nullptr) t *= 1.f / (1.f + expf(-(g[row * g_stride + i] + (g_bias != nullptr ? g_bias[i] : 0.f))));
+    const float s = fmaf(alpha, xr[i], t);
+    xr[i] = s;
+    ss += s * s;
+  }
+  const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = weight[i] * (xr[i] * r);
+    xr[i] = v;
+    if (rounded != nullptr) rounded[row * width + i] = from_f32<R>(v);
+  }
+}
+
 __global__ void softcap_kernel(float* __restrict__ y, int64_t n, float cap) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) y[i] = cap * tanhf(y[i] / cap);
@@ -127,7 +154,7 @@ __global__ void token_shift_kernel(const float* __restrict__ x, const float* __r
 // act: 0 none, 1 tanh. t is [rows][t_stride] (rank values a row), w2t [rank][features] (the matrix
 // transposed, so that neighbouring threads read neighbouring weights), out [rows][features].
 // out_act: what becomes of y before it is stored: 0 y itself; 1 exp(-exp(-1/2) sigmoid(y)) and
-// 2 exp(-exp(y)), the decays of the two recurrences. rate (may be nullptr): [rows][rate_stride], with
+// 2 exp(-exp(y)), the decays of the two recurrences; 3 softplus(y), a step size. rate (may be nullptr): [rows][rate_stride], with
 // features values a row that become sigmoid(rate + rate_bias) in place (the delta rule's removal
 // rate, made here because a thread a (row, feature) is what this launch already has).
 __global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride, const float* __restrict__ w2t,
@@ -157,6 +184,7 @@ __global__ void lowrank_out_kernel(const float* __restrict__ t, int64_t t_stride
   float y = ((s0 + s1) + (s2 + s3)) + (bias != nullptr ? bias[c] : 0.f);
   if (out_act == 1) y = expf(-0.6065306597126334f / (1.f + expf(-y)));
   else if (out_act == 2) y = expf(-expf(y));
+  else if (out_act == 3) y = y > 20.f ? y : log1pf(expf(y));
   out[row * features + c] = y;
   if (rate != nullptr) {
     float* r = rate + row * rate_stride + c;
@@ -379,6 +407,21 @@ int dli_rms_norm_from_f32(const float* x, const float* weight, void* out, int ro
   return dli_launch_status();
 }
 
+int dli_post_norm_stream(const void* y, int64_t y_stride, const float* g, int64_t g_stride, const float* g_bias,
+                         const float* weight, float* x, void* rounded_bf16, int rows, int width, float alpha, float eps,
+                         int y_is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0 || y_stride < width || (g != nullptr && g_stride < width)) return DLI_ERR_ARGUMENT;
+  const int threads = width >= 2048 ? 512 : 256;
+  if (y_is_bf16)
+    post_norm_stream_kernel<bf16_t, bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)y, y_stride, g, g_stride, g_bias,
+                                                                          weight, x, (bf16_t*)rounded_bf16, width, alpha, eps);
+  else
+    post_norm_stream_kernel<float, bf16_t><<<rows, threads, 0, stream>>>((const float*)y, y_stride, g, g_stride, g_bias,
+                                                                         weight, x, (bf16_t*)rounded_bf16, width, alpha, eps);
+  return dli_launch_status();
+}
+
 int dli_softcap(float* y, int64_t n, float cap, hipStream_t stream) {
   if (n <= 0) return DLI_OK;
   const int64_t blocks = (n + 255) / 256;
@@ -406,7 +449,7 @@ int dli_lowrank_out(const float* t, int64_t t_stride, const float* w2t, const fl
                     int features, int rank, int act, int out_act, float* rate, int64_t rate_stride,
                     const float* rate_bias, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
-  if (features <= 0 || rank <= 0 || rank > 8192 || t_stride < rank || act < 0 || act > 1 || out_act < 0 || out_act > 2 ||
+  if (features <= 0 || rank <= 0 || rank > 8192 || t_stride < rank || act < 0 || act > 1 || out_act < 0 || out_act > 3 ||
       (rate != nullptr && rate_stride < features))
     return DLI_ERR_ARGUMENT;
   lowrank_out_kernel<<<dim3(rows, (features + 255) / 256), 256, rank * sizeof(float), stream>>>(t, t_stride, w2t, bias, out,

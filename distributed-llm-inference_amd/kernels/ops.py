@@ -109,6 +109,21 @@ _SIGNATURES = {
     "dli_norm_into_stream": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_rms_norm_from_f32": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_softcap": [_c_ptr, _c_i64, _c_float, _c_ptr],
+    "dli_post_norm_stream": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float,
+                             _c_float, _c_int, _c_ptr],
+    "dli_causal_conv": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64,
+                        _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_selective_scan_max_states": [],
+    "dli_selective_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr, _c_ptr,
+                           _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int,
+                           _c_ptr],
+    "dli_bounded_gates": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
+    "dli_gated_linear_scan": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
+                              _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_latent_norm_cache": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_ptr,
+                              _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_head_products": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int,
+                          _c_ptr],
     "dli_token_shift": [_c_ptr, _c_ptr, _c_int, _c_ptr, _c_i64, _c_ptr, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
                         _c_int, _c_ptr],
     "dli_lowrank_out": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_i64,
@@ -131,11 +146,13 @@ _SIGNATURES = {
     "dli_gated_delta_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int,
                              _c_int, _c_int, _c_int, _c_ptr],
     "dli_poly_norm": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_float, _c_int, _c_ptr],
-    "dli_clamped_glu": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
-    "dli_router_choose": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr, _c_ptr],
+    "dli_clamped_glu": [_c_ptr, _c_i64, _c_ptr, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int, _c_ptr],
+    "dli_router_choose": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_ptr,
+                          _c_ptr],
     "dli_expert_tile_rows": [_c_int, _c_int, _c_int],
     "dli_expert_products": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int,
-                            _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_ptr],
+                            _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_float, _c_int,
+                            _c_ptr],
     "dli_expert_combine": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_int, _c_int,
                            _c_int, _c_int, _c_int, _c_ptr],
 }
@@ -1405,6 +1422,33 @@ def norm_into_stream(y: torch.Tensor, weight: torch.Tensor, eps: float, x: torch
                                           float(eps), _is_bf16(y.dtype), _stream()), "norm_into_stream")
 
 
+def post_norm_stream(x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, alpha: float, eps: float,
+                     gate: Optional[torch.Tensor] = None, gate_bias: Optional[torch.Tensor] = None,
+                     rounded: Optional[torch.Tensor] = None) -> None:
+    """``x <- weight * s / sqrt(mean(s^2) + eps)`` with ``s = alpha x + r y`` row by row, where
+    ``r = sigmoid(gate + gate_bias)`` element by element (``gate`` float32 ``[n, width]``, rows contiguous;
+    ``None``: ``r = 1``): the norm after a residual sum. ``x`` float32 ``[n, width]``, ``y`` float32 or bfloat16
+    with contiguous rows; sums and statistics in 32-bit. ``rounded``: the new ``x`` once more in bfloat16."""
+    _rounded_copy(rounded, x)
+    _rows(y, "y", y.dtype)
+    _dense(x, "x", torch.float32, 2)
+    _dense(weight, "weight", torch.float32, 1)
+    _require(y.shape == x.shape and weight.shape[0] == x.shape[1], "y, x and weight disagree on the sizes")
+    g_stride = 0
+    if gate is not None:
+        _f32_rows(gate, "gate")
+        _require(gate.shape == x.shape, "gate differs from x in shape")
+        g_stride = gate.stride(0)
+        if gate_bias is not None:
+            _dense(gate_bias, "gate_bias", torch.float32, 1)
+            _require(gate_bias.shape[0] == x.shape[1], "gate_bias must hold a value per column")
+    else:
+        _require(gate_bias is None, "a gate's bias comes with a gate")
+    _check(library().dli_post_norm_stream(_ptr(y), y.stride(0), _ptr(gate), g_stride, _ptr(gate_bias), _ptr(weight), _ptr(x),
+                                          _ptr(rounded), x.shape[0], x.shape[1], float(alpha), float(eps),
+                                          _is_bf16(y.dtype), _stream()), "post_norm_stream")
+
+
 def rms_norm_from_f32(x: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
     """``out = weight * x / sqrt(mean(x^2) + eps)`` for a float32 ``x``, rounded once to ``out``'s type."""
     _dense(x, "x", torch.float32, 2)
@@ -1444,7 +1488,7 @@ def token_shift(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, q_start:
                                      _is_bf16(out.dtype), _stream()), "token_shift")
 
 
-LOWRANK_OUT_ACTS = {"none": 0, "delta_decay": 1, "double_exp_decay": 2}
+LOWRANK_OUT_ACTS = {"none": 0, "delta_decay": 1, "double_exp_decay": 2, "softplus": 3}
 
 
 def lowrank_out(t: torch.Tensor, w2t: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
@@ -1807,21 +1851,28 @@ def gated_delta_scan(prep: torch.Tensor, state: torch.Tensor, q_start: torch.Ten
         _ptr(o), o.stride(0), entries, n, heads, kv_heads, dim, vdim, _stream()), "gated_delta_scan")
 
 
-def head_norm_gate(o: torch.Tensor, g_pre: torch.Tensor, norm_w: torch.Tensor, eps: float, out: torch.Tensor,
+HEAD_GATES = {"sigmoid": 0, "silu": 1, "none": 2}
+
+
+def head_norm_gate(o: torch.Tensor, g_pre: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float, out: torch.Tensor,
                    heads: int, dim: int, gate: str = "silu") -> None:
     """``out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre)`` head by head: ``o`` and ``g_pre`` float32
-    ``[n, heads*dim]`` (rows contiguous), ``norm_w`` float32 ``[heads*dim]``, ``gate`` ``"silu"`` or ``"sigmoid"``."""
+    ``[n, heads*dim]`` (rows contiguous), ``norm_w`` float32 ``[heads*dim]``, ``gate`` ``"silu"``, ``"sigmoid"`` or
+    ``"none"`` (the per-head norm alone; ``g_pre`` is then ``None``)."""
     _f32_rows(o, "o")
-    _f32_rows(g_pre, "g_pre")
     _rows(out, "out", out.dtype)
     _dense(norm_w, "norm_w", torch.float32, 1)
     n, width = o.shape[0], heads * dim
-    _require(o.shape == (n, width) and g_pre.shape == (n, width) and out.shape == (n, width) and norm_w.shape[0] == width,
-             "o, g_pre, out and norm_w must be [n, heads*dim]")
-    _require(gate in ("silu", "sigmoid"), "gate must be 'silu' or 'sigmoid'")
-    _check(library().dli_head_norm_gate(_ptr(o), o.stride(0), _ptr(g_pre), g_pre.stride(0), _ptr(norm_w), float(eps),
-                                        _ptr(out), out.stride(0), n, heads, dim, int(gate == "silu"),
-                                        _is_bf16(out.dtype), _stream()), "head_norm_gate")
+    _require(gate in HEAD_GATES, f"gate must be one of {sorted(HEAD_GATES)}")
+    _require((g_pre is None) == (gate == "none"), "g_pre comes with a gate, and only with one")
+    if g_pre is not None:
+        _f32_rows(g_pre, "g_pre")
+        _require(g_pre.shape == (n, width), "g_pre must be [n, heads*dim]")
+    _require(o.shape == (n, width) and out.shape == (n, width) and norm_w.shape[0] == width,
+             "o, out and norm_w must be [n, heads*dim]")
+    _check(library().dli_head_norm_gate(_ptr(o), o.stride(0), _ptr(g_pre), 0 if g_pre is None else g_pre.stride(0),
+                                        _ptr(norm_w), float(eps), _ptr(out), out.stride(0), n, heads, dim,
+                                        HEAD_GATES[gate], _is_bf16(out.dtype), _stream()), "head_norm_gate")
 
 
 # ----------------------------------------------------------------------------- feed-forward: polynomial activation, experts
@@ -1837,21 +1888,22 @@ def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor
                                    float(eps), _is_bf16(out.dtype), _stream()), "poly_norm")
 
 
-def clamped_glu(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float) -> None:
-    """``out = g sigmoid(alpha g) (u + 1)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``;
+def clamped_glu(gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float, up_shift: float = 1.0) -> None:
+    """``out = g sigmoid(alpha g) (u + up_shift)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``
+    (an infinite limit, ``alpha = 1`` and ``up_shift = 0``: ``silu(gate) * up``);
     ``gate_up [n, >= 2 ff]`` holds gate then up (rows contiguous), ``out [n, ff]`` of the same type."""
     _rows(gate_up, "gate_up", out.dtype)
     _dense(out, "out", ndim=2)
     n, ff = out.shape
     _require(gate_up.shape[0] == n and gate_up.shape[1] >= 2 * ff, "gate_up must hold gate and up for every row")
     _check(library().dli_clamped_glu(_ptr(gate_up), gate_up.stride(0), _ptr(out), n, ff, float(limit), float(alpha),
-                                     _is_bf16(out.dtype), _stream()), "clamped_glu")
+                                     float(up_shift), _is_bf16(out.dtype), _stream()), "clamped_glu")
 
 
 def router_choose(logits: torch.Tensor, total: int, correction: Optional[torch.Tensor], groups: int, keep: int, top: int,
-                  scale: float, ids: torch.Tensor, weights: torch.Tensor) -> None:
+                  scale: float, ids: torch.Tensor, weights: torch.Tensor, bias: Optional[torch.Tensor] = None) -> None:
     """The router's choice per row of float32 ``logits [n, >= total]``: scores ``softmax`` over the first
-    ``total`` columns; choice scores add ``correction``; with ``groups`` > 1 only the ``keep`` groups of
+    ``total`` columns (plus ``bias``, float32 ``[total]``, where the router has one); choice scores add ``correction``; with ``groups`` > 1 only the ``keep`` groups of
     neighbours with the largest best choice score can be chosen; ``ids [n, top]`` int32 are the largest
     choice scores (lowest index on a tie), ``weights [n, top]`` their scores (without correction) divided
     by their sum + 1e-20, times ``scale``."""
@@ -1861,18 +1913,21 @@ def router_choose(logits: torch.Tensor, total: int, correction: Optional[torch.T
     if correction is not None:
         _dense(correction, "correction", torch.float32, 1)
         _require(correction.shape[0] == total, "correction must hold a value per router output")
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] == total, "bias must hold a value per router output")
     _dense(ids, "ids", torch.int32, 2)
     _dense(weights, "weights", torch.float32, 2)
     _require(ids.shape == (n, top) and weights.shape == (n, top), "ids and weights must be [n, top]")
     _require(1 <= top <= min(total, 64) and groups >= 1 and total % groups == 0 and 1 <= keep <= groups
              and keep * (total // groups) >= top, "the router's sizes do not fit each other")
-    _check(library().dli_router_choose(_ptr(logits), logits.stride(0), _ptr(correction), n, int(total), int(groups),
+    _check(library().dli_router_choose(_ptr(logits), logits.stride(0), _ptr(bias), _ptr(correction), n, int(total), int(groups),
                                        int(keep), int(top), float(scale), _ptr(ids), _ptr(weights), _stream()),
            "router_choose")
 
 
 def expert_products(ids: torch.Tensor, h: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
-                    limit: float, alpha: float) -> torch.Tensor:
+                    limit: float, alpha: float, up_shift: float = 1.0) -> torch.Tensor:
     """The chosen experts' results for every (token, choice): ``z [n * top, width]`` float32, row
     ``t * top + j`` holding ``w_down[e] clamped_glu(w_gate[e] h_t, w_up[e] h_t)`` for ``e = ids[t, j]`` (rows of
     ids at or above the number of experts are left unwritten). ``w_gate, w_up [experts, ff, width]``,
@@ -1898,7 +1953,7 @@ def expert_products(ids: torch.Tensor, h: torch.Tensor, w_gate: torch.Tensor, w_
     _check(library().dli_expert_products(
         _ptr(ids), _ptr(h), h.stride(0), _ptr(w_gate), _ptr(w_up), _ptr(w_down), _ptr(offsets), _ptr(order),
         _ptr(tile_expert), _ptr(tile_row0), _ptr(tile_count), max_tiles, _ptr(y), _ptr(z), n, top, experts, width, ff,
-        float(limit), float(alpha), _is_bf16(h.dtype), _stream()), "expert_products")
+        float(limit), float(alpha), float(up_shift), _is_bf16(h.dtype), _stream()), "expert_products")
     return z
 
 
@@ -1932,3 +1987,182 @@ def expert_combine(ids: torch.Tensor, weights: torch.Tensor, z: Optional[torch.T
     _check(library().dli_expert_combine(_ptr(ids), _ptr(weights), _ptr(z), _ptr(h), h.stride(0), _ptr(shared_gate), g_stride,
                                         _ptr(shared), s_stride, _ptr(out), n, top, int(experts), width, _is_bf16(h.dtype),
                                         _stream()), "expert_combine")
+
+
+# ----------------------------------------------------------------------------- short convolutions, the selective scan
+
+def _step_arrays(q_start: torch.Tensor, positions: torch.Tensor, state_slots: torch.Tensor, n: int) -> int:
+    for name, t in (("q_start", q_start), ("positions", positions), ("state_slots", state_slots)):
+        _dense(t, name, torch.int32, 1)
+    entries = state_slots.shape[0]
+    _require(q_start.shape[0] == entries + 1 and positions.shape[0] == n, "q_start/state_slots/positions disagree")
+    return entries
+
+
+def _state_rows(state: torch.Tensor, floats: int) -> None:
+    _require(state.is_cuda and state.dtype == torch.float32 and state.dim() == 2 and state.stride(1) == 1
+             and state.shape[1] >= floats, f"state must be float32 [slots, >= {floats}]")
+
+
+def causal_conv(x: torch.Tensor, conv_w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor, kept_offset: int,
+                q_start: torch.Tensor, positions: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor,
+                rounded: Optional[torch.Tensor] = None, act: str = "silu") -> None:
+    """A short causal convolution over time per channel: ``out[t, c] = act(bias[c] + sum_j conv_w[c, taps-1-j] x[t-j, c])``
+    with zeros before position 0. ``x`` float32 ``[n, >= channels]`` (rows contiguous; the channels from
+    column 0), ``conv_w`` float32 ``[channels, taps]`` (the last column is the current token's). The inputs
+    before an entry's first row come from ``state[slot, kept_offset:]`` (``[taps-1, channels]``, the newest
+    last), which then receives the entry's last ``taps - 1`` inputs. ``out`` float32 ``[n, channels]``;
+    ``rounded``: the result once more (float32 or bfloat16), for the product that reads it next.
+    ``act``: ``"silu"`` or ``"none"``."""
+    _f32_rows(x, "x")
+    _dense(conv_w, "conv_w", torch.float32, 2)
+    channels, taps = conv_w.shape
+    n = x.shape[0]
+    _require(x.shape[1] >= channels, "x must hold every channel")
+    _require(1 <= taps <= gated_delta_max_taps(), "too many taps")
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] == channels, "bias must hold a value per channel")
+    _f32_rows(out, "out")
+    _require(out.shape == (n, channels), "out must be [n, channels]")
+    r_stride, r_bf16 = 0, 0
+    if rounded is not None:
+        _rows(rounded, "rounded", rounded.dtype)
+        _require(rounded.shape == (n, channels), "the rounded copy must be [n, channels]")
+        r_stride, r_bf16 = rounded.stride(0), _is_bf16(rounded.dtype)
+    _require(act in ("silu", "none"), "act must be 'silu' or 'none'")
+    _state_rows(state, kept_offset + (taps - 1) * channels)
+    entries = _step_arrays(q_start, positions, state_slots, n)
+    _check(library().dli_causal_conv(
+        _ptr(x), x.stride(0), _ptr(conv_w), _ptr(bias), _ptr(state), state.stride(0), int(kept_offset), _ptr(q_start),
+        _ptr(positions), _ptr(state_slots), _ptr(out), out.stride(0), _ptr(rounded), r_stride, r_bf16, entries, n,
+        channels, taps, int(act == "silu"), _stream()), "causal_conv")
+
+
+def selective_scan_max_states() -> int:
+    return int(library().dli_selective_scan_max_states())
+
+
+def selective_scan(x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, b_off: int, c_off: int, z: Optional[torch.Tensor],
+                   a_log: torch.Tensor, d: Optional[torch.Tensor], state: torch.Tensor, q_start: torch.Tensor,
+                   positions: torch.Tensor, state_slots: torch.Tensor, out: torch.Tensor) -> None:
+    """Per request and channel ``S[n] <- exp(dt A[n]) S[n] + dt x B[n]``, ``y = sum_n S[n] C[n] + d x``,
+    ``out = y silu(z)`` over the step's rows in order, ``A = -exp(a_log)``. ``x``, ``dt`` (positive step sizes)
+    and ``z`` (``None``: no gate) float32 ``[n, channels]`` (rows contiguous), ``bc`` float32 ``[n, >=]`` with the
+    token's B and C (``states`` values each) at columns ``b_off`` and ``c_off``, ``a_log`` float32
+    ``[channels, states]``, ``d`` float32 ``[channels]`` or ``None``. ``S`` float32 ``[channels][states]`` at
+    the start of ``state[slot]`` (zeros at position 0). ``out [n, channels]``, float32 or bfloat16."""
+    _f32_rows(x, "x")
+    _f32_rows(dt, "dt")
+    _f32_rows(bc, "bc")
+    _dense(a_log, "a_log", torch.float32, 2)
+    channels, states = a_log.shape
+    n = x.shape[0]
+    _require(x.shape == (n, channels) and dt.shape == (n, channels), "x and dt must be [n, channels]")
+    _require(1 <= states <= selective_scan_max_states(), "too many states a channel")
+    _require(bc.shape[0] == n and 0 <= b_off and b_off + states <= bc.shape[1] and 0 <= c_off
+             and c_off + states <= bc.shape[1], "B or C lie outside bc")
+    if z is not None:
+        _f32_rows(z, "z")
+        _require(z.shape == (n, channels), "z must be [n, channels]")
+    if d is not None:
+        _dense(d, "d", torch.float32, 1)
+        _require(d.shape[0] == channels, "d must hold a value per channel")
+    _rows(out, "out", out.dtype)
+    _require(out.shape == (n, channels), "out must be [n, channels]")
+    _state_rows(state, channels * states)
+    entries = _step_arrays(q_start, positions, state_slots, n)
+    _check(library().dli_selective_scan(
+        _ptr(x), x.stride(0), _ptr(dt), dt.stride(0), _ptr(bc), bc.stride(0), int(b_off), int(c_off), _ptr(z),
+        0 if z is None else z.stride(0), _ptr(a_log), _ptr(d), _ptr(state), state.stride(0), _ptr(q_start), _ptr(positions),
+        _ptr(state_slots), _ptr(out), out.stride(0), entries, n, channels, states, _is_bf16(out.dtype), _stream()),
+        "selective_scan")
+
+
+# ----------------------------------------------------------------------------- the gated linear recurrence
+
+def bounded_gates(proj: torch.Tensor, q_off: int, f_off: int, width: int, f_bias: Optional[torch.Tensor],
+                  lower: Optional[torch.Tensor]) -> None:
+    """In place on float32 ``proj [n, >=]``: the ``width`` columns from ``q_off`` become ``silu`` of themselves,
+    those from ``f_off`` become ``lower + (1 - lower) sigmoid(. + f_bias)`` (``lower``, ``f_bias`` float32
+    ``[width]``; ``None``: zeros)."""
+    _f32_rows(proj, "proj")
+    for name, t in (("f_bias", f_bias), ("lower", lower)):
+        if t is not None:
+            _dense(t, name, torch.float32, 1)
+            _require(t.shape[0] == width, f"{name} must hold a value per column")
+    _require(0 <= q_off and q_off + width <= proj.shape[1] and 0 <= f_off and f_off + width <= proj.shape[1]
+             and (q_off + width <= f_off or f_off + width <= q_off), "the columns lie outside proj or overlap")
+    _check(library().dli_bounded_gates(_ptr(proj), proj.stride(0), int(q_off), int(f_off), _ptr(f_bias), _ptr(lower),
+                                       proj.shape[0], int(width), _stream()), "bounded_gates")
+
+
+def gated_linear_scan(proj: torch.Tensor, q_off: int, f_off: int, v_off: int, state: torch.Tensor, q_start: torch.Tensor,
+                      positions: torch.Tensor, state_slots: torch.Tensor, o: torch.Tensor, heads: int, dim: int,
+                      vdim: int) -> None:
+    """Per request and head ``S <- diag(f) S + (1 - f) v^T``, ``o = S^T q`` over the step's rows in order:
+    float32 ``proj [n, >=]`` holds q and f (``heads x dim`` each, as :func:`bounded_gates` leaves them) and v
+    (``heads x vdim``) at their columns; ``S`` float32 ``[heads][vdim][dim]`` at the start of ``state[slot]``
+    (zeros at position 0); ``o [n, heads*vdim]`` float32."""
+    _f32_rows(proj, "proj")
+    _f32_rows(o, "o")
+    n = proj.shape[0]
+    _require(o.shape == (n, heads * vdim), "o must be [n, heads*vdim]")
+    _require(all(0 <= off and off + heads * size <= proj.shape[1]
+                 for off, size in ((q_off, dim), (f_off, dim), (v_off, vdim))), "q, f or v lie outside proj")
+    _state_rows(state, heads * vdim * dim)
+    entries = _step_arrays(q_start, positions, state_slots, n)
+    _check(library().dli_gated_linear_scan(
+        _ptr(proj), proj.stride(0), int(q_off), int(f_off), int(v_off), _ptr(state), state.stride(0), _ptr(q_start),
+        _ptr(positions), _ptr(state_slots), _ptr(o), o.stride(0), entries, n, heads, dim, vdim, _stream()),
+        "gated_linear_scan")
+
+
+# ----------------------------------------------------------------------------- attention through a latent
+
+def latent_norm_cache(proj: torch.Tensor, q_off: int, q_rank: int, c_off: int, rank: int, q_weight: torch.Tensor,
+                      c_weight: torch.Tensor, eps: float, q_out: torch.Tensor, slots: torch.Tensor, k_pages: torch.Tensor,
+                      v_pages: torch.Tensor) -> None:
+    """From float32 ``proj [n, >=]``: the ``q_rank`` columns from ``q_off`` and the ``rank`` columns from ``c_off``
+    each divided by their root mean square (eps inside the root) and multiplied by their weight; the first
+    goes to ``q_out [n, q_rank]``, the second into the token's cache slot (negative: not cached) as a key,
+    ``k_pages [pages, 1, page_size, rank]``, and as a value, ``v_pages [pages, 1, rank, page_size]``."""
+    _f32_rows(proj, "proj")
+    n = proj.shape[0]
+    _dense(q_weight, "q_weight", torch.float32, 1)
+    _dense(c_weight, "c_weight", torch.float32, 1)
+    _require(q_weight.shape[0] == q_rank and c_weight.shape[0] == rank, "the weights must fit the latents")
+    _require(0 <= q_off and q_off + q_rank <= proj.shape[1] and 0 <= c_off and c_off + rank <= proj.shape[1],
+             "the latents lie outside proj")
+    _dense(q_out, "q_out", ndim=2)
+    _require(q_out.shape == (n, q_rank), "q_out must be [n, q_rank]")
+    _dense(k_pages, "k_pages", q_out.dtype, 4)
+    _dense(v_pages, "v_pages", q_out.dtype, 4)
+    pages, _, page_size, _ = k_pages.shape
+    _require(k_pages.shape == (pages, 1, page_size, rank) and v_pages.shape == (pages, 1, rank, page_size),
+             "the pages must hold one latent a token: k [pages, 1, page_size, rank], v [pages, 1, rank, page_size]")
+    _dense(slots, "slots", torch.int32, 1)
+    _require(slots.shape[0] == n, "a cache slot per row")
+    _check(library().dli_latent_norm_cache(
+        _ptr(proj), proj.stride(0), int(q_off), int(q_rank), int(c_off), int(rank), _ptr(q_weight), _ptr(c_weight),
+        float(eps), _ptr(q_out), _ptr(slots), _ptr(k_pages), _ptr(v_pages), n, page_size, _is_bf16(q_out.dtype),
+        _stream()), "latent_norm_cache")
+
+
+def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Optional[torch.Tensor] = None) -> None:
+    """``out[t, h] = w[h] x[t, h]`` for every head (32-bit sums, ascending k): ``x [n, heads*k]``,
+    ``w [heads, m, k]``, ``out [n, heads*m]``, all of one type (float32 or bfloat16, rows contiguous);
+    ``gate`` (float32 ``[n, heads*m]``): the result is multiplied by its sigmoid."""
+    _dense(w, "w", ndim=3)
+    heads, m, k = w.shape
+    _rows(x, "x", w.dtype)
+    _rows(out, "out", w.dtype)
+    n = x.shape[0]
+    _require(x.shape == (n, heads * k) and out.shape == (n, heads * m), "x must be [n, heads*k] and out [n, heads*m]")
+    g_stride = 0
+    if gate is not None:
+        _f32_rows(gate, "gate")
+        _require(gate.shape == out.shape, "gate differs from out in shape")
+        g_stride = gate.stride(0)
+    _check(library().dli_head_products(_ptr(x), x.stride(0), _ptr(w), _ptr(out), out.stride(0), _ptr(gate), g_stride, n,
+                                       heads, m, k, _is_bf16(w.dtype), _stream()), "head_products")

@@ -104,3 +104,71 @@ class OutputNormBlock(Block):
             y = parts["feed_forward"].forward(as_operand(self.rt, x, ctx), ctx)
             parts["feed_forward_norm"].add_normed(x, y, ctx)
         return x, None
+
+
+@register_part("block", "post_norm")
+class PostNormBlock(Block):
+    """Norms after the residual sums, around a 32-bit residual stream:
+    ``x <- norm1(alpha x + r1 * mixer(x))``, then ``x <- norm2(alpha x + r2 * feed_forward(x))``; the sublayers
+    read ``x`` itself. With ``gated`` each sublayer's result is multiplied element by element by
+    ``r = sigmoid(W x + b)`` before the sum (tensors ``rg1``, ``rg1.b`` for the mixer and ``rg2``, ``rg2.b`` for
+    the feed-forward, below this block's prefix; ``W`` reads the same ``x`` as the sublayer); without,
+    ``r = 1``. The feed-forward and its norm may be absent. ``x`` is float32 in both runtimes; gate, sum and
+    norm are one kernel (``Norm.post_norm``). The mixer gets the stream as it is (what it feeds to its
+    products it rounds itself); the feed-forward gets it in the type that its products read."""
+
+    roles = ("mixer", "mixer_norm")
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, alpha: float = 1.0, gated: bool = False,
+                 feed_forward: bool = True, names: Optional[Mapping[str, str]] = None) -> None:
+        super().__init__(runtime)
+        self.hidden_size, self.alpha, self.gated, self.has_ff = hidden_size, float(alpha), bool(gated), bool(feed_forward)
+        self.names = {"mixer": "rg1", "feed_forward": "rg2", **dict(names or {})}
+        self.w: dict[str, torch.Tensor] = {}
+        self.b: dict[str, torch.Tensor] = {}
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
+    def _gates(self) -> list[str]:
+        return [] if not self.gated else ["mixer"] + (["feed_forward"] if self.has_ff else [])
+
+    def weight_specs(self) -> dict:
+        from .spec import WeightSpec
+
+        h, specs = self.hidden_size, {}
+        for role in self._gates():
+            specs[self.names[role]] = WeightSpec((h, h))
+            specs[self.names[role] + ".b"] = WeightSpec((h,), role="float32", init="zeros")
+        return specs
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        for role in self._gates():
+            self.w[role] = tensors[self.names[role]]
+            self.b[role] = tensors[self.names[role] + ".b"].contiguous()
+
+    def _gate(self, role: str, operand: torch.Tensor) -> tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+        if not self.gated:
+            return None, None
+        from .linear import linear_f32
+
+        return linear_f32(self.rt, operand, self.w[role]), self.b[role]
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
+                parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
+        if x.dtype != torch.float32:
+            raise RuntimeError("the post_norm block keeps a float32 residual stream")
+        if delta is not None:
+            from ..kernels import ops
+            from .linear import RoundedStream
+            ops.add(x, delta, x)
+            RoundedStream.offer(ctx, x, None)
+        g, b = self._gate("mixer", as_operand(self.rt, x, ctx))
+        y = parts["mixer"].forward(x, ctx, cache)
+        parts["mixer_norm"].post_norm(x, y, self.alpha, ctx, gate=g, gate_bias=b)
+        if "feed_forward" in parts:
+            h = as_operand(self.rt, x, ctx)
+            g, b = self._gate("feed_forward", h)
+            y = parts["feed_forward"].forward(h, ctx)
+            parts["feed_forward_norm"].post_norm(x, y, self.alpha, ctx, gate=g, gate_bias=b)
+        return x, None

@@ -1,16 +1,19 @@
 """A mixture of small feed-forward experts behind a router.
 
-Router: ``z = W_router h`` in 32-bit over ``experts + identity`` outputs, scores ``s = softmax(z)``. The
+Router: ``z = W_router h`` (``+ b_router`` with ``router_bias``) in 32-bit over ``experts + identity`` outputs, scores
+``s = softmax(z)``. The
 choice scores add a per-output ``correction`` (the weights do not). The outputs form ``groups`` equal
 groups of neighbours; a group's score is its largest choice score, and only outputs of the best
 ``groups_kept`` groups can be chosen. The ``top`` largest choice scores are chosen; their weights are
-their scores ``s`` divided by their sum (+ 1e-20), times ``scale``. The last ``identity`` outputs are
+their scores ``s`` divided by their sum (+ 1e-20), times ``scale`` (with ``scale = 1`` and without correction and
+groups that is the softmax over the chosen logits alone). The last ``identity`` outputs are
 identity experts: their result is the input itself; they have no tensors.
 
 Expert ``e`` (tensors ``e<e>.gate``, ``e<e>.up``, ``e<e>.down``, no biases): ``g = min(W_gate h, limit)``,
-``u = clamp(W_up h, -limit, limit)``, ``y = g sigmoid(alpha g) (u + 1)``, result ``W_down y``. A shared
+``u = clamp(W_up h, -limit, limit)``, ``y = g sigmoid(alpha g) (u + up_shift)``, result ``W_down y`` (an infinite
+limit, ``alpha = 1`` and ``up_shift = 0``: the plain ``silu(W_gate h) * (W_up h)``). A shared
 expert of the same form (its own size and limit) may run for every token; it is added multiplied by
-``sigmoid(W_sg h)``, one number per token.
+``sigmoid(W_sg h)``, one number per token, or as it is (``shared_gate=False``).
 
 Order of work: one 32-bit product for the router (and the shared expert's gate: its row is stacked
 below the router's); the choice kernel; on the device the chosen (token, expert) pairs are sorted by
@@ -37,7 +40,7 @@ class RoutedExperts(FeedForward):
     def __init__(self, runtime: Runtime, *, hidden_size: int, experts: int, top: int, expert_size: int,
                  limit: float, alpha: float = 1.702, identity: int = 0, groups: int = 1, groups_kept: int = 1,
                  scale: float = 1.0, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0,
-                 shared_gate: bool = True) -> None:
+                 shared_gate: bool = True, up_shift: float = 1.0, router_bias: bool = False) -> None:
         super().__init__(runtime)
         total = experts + identity
         if experts < 0 or identity < 0 or total < 1 or not 1 <= top <= min(total, 64):
@@ -49,10 +52,10 @@ class RoutedExperts(FeedForward):
         self.hidden_size, self.experts, self.identity, self.total, self.top = hidden_size, experts, identity, total, top
         self.expert_size, self.limit, self.alpha = expert_size, float(limit), float(alpha)
         self.groups, self.groups_kept, self.scale = groups, groups_kept, float(scale)
-        self.has_correction = bool(correction)
+        self.has_correction, self.has_router_bias, self.up_shift = bool(correction), bool(router_bias), float(up_shift)
         self.shared_size, self.shared_limit = int(shared_size), float(shared_limit)
         self.shared_gate = bool(shared_gate) and self.shared_size > 0
-        self.w_router = self.correction = self.w_gate = self.w_up = self.w_down = None
+        self.w_router = self.router_bias = self.correction = self.w_gate = self.w_up = self.w_down = None
         self.ws_gate_up = self.ws_down = None
 
     def graph_capturable(self, page_size: int) -> bool:
@@ -61,6 +64,8 @@ class RoutedExperts(FeedForward):
     def weight_specs(self) -> dict[str, WeightSpec]:
         h, f = self.hidden_size, self.expert_size
         specs = {"router": WeightSpec((self.total, h))}
+        if self.has_router_bias:
+            specs["router.b"] = WeightSpec((self.total,), role="float32", init="zeros")
         if self.has_correction:
             specs["correction"] = WeightSpec((self.total,), role="float32", init="zeros", optional=True)
         for e in range(self.experts):
@@ -75,6 +80,7 @@ class RoutedExperts(FeedForward):
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         rows = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_gate else [])
         self.w_router = stack_rows(rows)
+        self.router_bias = tensors["router.b"].contiguous() if self.has_router_bias else None
         # (a checkpoint without the tensor: scores are chosen as they are)
         self.correction = tensors["correction"].contiguous() if self.has_correction and "correction" in tensors else None
         if self.experts:
@@ -90,15 +96,16 @@ class RoutedExperts(FeedForward):
         logits = linear_f32(self.rt, x, self.w_router)
         ids = torch.empty(n, self.top, device=dev, dtype=torch.int32)
         weights = torch.empty(n, self.top, device=dev, dtype=torch.float32)
-        ops.router_choose(logits, self.total, self.correction, self.groups, self.groups_kept, self.top, self.scale, ids, weights)
+        ops.router_choose(logits, self.total, self.correction, self.groups, self.groups_kept, self.top, self.scale, ids, weights,
+                          bias=self.router_bias)
         z = None
         if self.experts:
-            z = ops.expert_products(ids, x, self.w_gate, self.w_up, self.w_down, self.limit, self.alpha)
+            z = ops.expert_products(ids, x, self.w_gate, self.w_up, self.w_down, self.limit, self.alpha, self.up_shift)
         shared = gate = None
         if self.shared_size:
             gate_up = linear(self.rt, x, self.ws_gate_up)
             act = self.rt.empty(n, self.shared_size)
-            ops.clamped_glu(gate_up, act, self.shared_limit, self.alpha)
+            ops.clamped_glu(gate_up, act, self.shared_limit, self.alpha, self.up_shift)
             shared = linear_f32(self.rt, act, self.ws_down)
             if self.shared_gate:
                 gate = logits[:, self.total:self.total + 1]

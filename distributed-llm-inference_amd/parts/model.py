@@ -21,7 +21,8 @@ from .spec import ModelSpec, WeightSpec
 
 # importing the modules registers the built-in parts
 from . import (  # noqa: F401,E402
-    attention, block, embedding, experts, feed_forward, head, norm, parallel, position, recurrent, scored_attention,
+    attention, block, embedding, experts, feed_forward, head, latent_attention, norm, parallel, position, recurrent,
+    scored_attention, selective_scan, token_shift,
 )
 
 

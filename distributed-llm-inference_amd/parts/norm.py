@@ -52,6 +52,18 @@ class RMSNorm(Norm):
         ops.norm_into_stream(y, self.weight, self.eps, x, rounded=rounded)
         RoundedStream.offer(ctx, x, rounded)
 
+    def post_norm(self, x: torch.Tensor, y: torch.Tensor, alpha: float, ctx=None, gate: Optional[torch.Tensor] = None,
+                  gate_bias: Optional[torch.Tensor] = None) -> None:
+        """``x <- norm(alpha x + r y)``, ``r = sigmoid(gate + gate_bias)`` or 1: the norm after a residual sum,
+        on a 32-bit residual stream ``x`` in one kernel (gate, sum, statistics and product in 32-bit; ``y``
+        float32 or bfloat16, ``gate`` float32). In a bfloat16 runtime the kernel leaves the new stream once
+        more in bfloat16 on ``ctx``, for the product that reads it next."""
+        from .linear import RoundedStream
+
+        rounded = self.rt.empty(*x.shape) if self.rt.is_bf16 and ctx is not None else None
+        ops.post_norm_stream(x, y, self.weight, alpha, self.eps, gate=gate, gate_bias=gate_bias, rounded=rounded)
+        RoundedStream.offer(ctx, x, rounded)
+
     def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor] = None) -> torch.Tensor:
         if x.dtype == torch.float32 and self.rt.is_bf16:
             # a 32-bit residual stream in a bfloat16 runtime: normalised in 32-bit and rounded once,

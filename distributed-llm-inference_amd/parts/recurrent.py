@@ -1,7 +1,8 @@
 """Mixers that carry a matrix state per head from token to token instead of a cache of keys:
 ``general_delta`` (a generalized delta rule), ``wkv`` (decayed sums with a bonus for the current
-token and token shift) and ``gated_delta`` (the delta rule with one decay and one write strength per
-head, behind short convolutions). The state lives in 32-bit in the request's state slot
+token and token shift), ``gated_delta`` (the delta rule with one decay and one write strength per
+head, behind short convolutions) and ``gated_linear`` (decayed sums whose forget gate also decides what
+is written). The state lives in 32-bit in the request's state slot
 (:class:`StateSpec`), starts at zero at position 0, and is all that a step leaves for the next.
 
 Both run their projections as products of the runtime's type with 32-bit sums, and everything
@@ -239,4 +240,58 @@ class GatedDelta(Mixer):
                              self.head_dim, self.value_dim)
         out = self.rt.empty(n, self.hv)
         ops.head_norm_gate(o, proj[:, g_off:g_off + self.hv], self.norm_w, self.norm_eps, out, H, self.value_dim, gate="silu")
+        return linear_f32(self.rt, out, self.w_o)
+
+
+@register_part("mixer", "gated_linear")
+class GatedLinear(Mixer):
+    """Linear attention in which the forget gate also decides what is written. From the rows ``h``:
+    ``q = silu(W_q h)`` (``num_heads x head_dim``), ``v = W_v h`` (``num_heads x value_dim``), and per head and key
+    channel the forget gate ``f = lower + (1 - lower) sigmoid(W_f h + b_f)`` with a lower bound per channel. Per
+    head ``S <- diag(f) S + (1 - f) v^T``, ``o = S^T q`` (no key, no scale); then each head's ``o / rms(o) * norm``
+    (``norm`` of ``value_dim`` values, shared by the heads) and the output product. The request's state slot
+    holds ``S`` in 32-bit; everything between the projections and the output product is 32-bit."""
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, head_dim: int, value_dim: Optional[int] = None,
+                 norm_eps: float = 1e-6) -> None:
+        super().__init__(runtime)
+        value_dim = head_dim if value_dim is None else value_dim
+        if min(hidden_size, num_heads, head_dim, value_dim) < 1:
+            raise ValueError("heads and their sizes must be positive")
+        self.hidden_size, self.num_heads, self.head_dim, self.value_dim = hidden_size, num_heads, head_dim, value_dim
+        self.norm_eps = float(norm_eps)
+        self.hd, self.hv = num_heads * head_dim, num_heads * value_dim
+        self.w_in = self.f_bias = self.lower = self.norm_w = self.w_o = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h = self.hidden_size
+        return {"q": WeightSpec((self.hd, h)), "f": WeightSpec((self.hd, h)),
+                "f.b": WeightSpec((self.hd,), role="float32", init="zeros"),
+                "lower": WeightSpec((self.hd,), role="float32", init="zeros"), "v": WeightSpec((self.hv, h)),
+                "norm": WeightSpec((self.value_dim,), role="float32", init="norm"), "o": WeightSpec((h, self.hv))}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_in = stack_rows([tensors[n] for n in ("q", "f", "v")])   # one product for everything that reads h
+        self.f_bias, self.lower = tensors["f.b"].contiguous(), tensors["lower"].contiguous()
+        self.norm_w = tensors["norm"].repeat(self.num_heads).contiguous()   # the kernel reads a value per head and column
+        self.w_o = tensors["o"]
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.num_heads * self.value_dim * self.head_dim,), torch.float32)
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on the context's device arrays only; padding rows write the spare slot
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any) -> torch.Tensor:
+        if cache is None or cache.kind != "state" or not cache.writable:
+            raise RuntimeError("gated_linear needs a state of its own")
+        state = cache.state.view(cache.state.shape[0], -1)
+        n = x.shape[0]
+        proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)         # q | f | v
+        ops.bounded_gates(proj, 0, self.hd, self.hd, self.f_bias, self.lower)
+        o = torch.empty(n, self.hv, device=self.rt.device, dtype=torch.float32)
+        ops.gated_linear_scan(proj, 0, self.hd, 2 * self.hd, state, ctx.q_start, ctx.positions, ctx.state_slots, o,
+                              self.num_heads, self.head_dim, self.value_dim)
+        out = self.rt.empty(n, self.hv)
+        ops.head_norm_gate(o, None, self.norm_w, self.norm_eps, out, self.num_heads, self.value_dim, gate="none")
         return linear_f32(self.rt, out, self.w_o)

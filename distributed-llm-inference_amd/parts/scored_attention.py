@@ -37,6 +37,34 @@ from .registry import build_part, register_part
 from .spec import PartSpec, WeightSpec
 
 
+def paged_scored_attention(rt: Runtime, ctx: Any, cache: Any, q: torch.Tensor, out: torch.Tensor, num_heads: int,
+                           head_dim: int, value_dim: int, scale: float, *, gate: Optional[torch.Tensor] = None,
+                           **changes: Any) -> None:
+    """The attention of a step's rows over a paged cache, for any mixer that has written its keys and
+    values there: steps of single tokens go to the kernel that reads the context's device arrays alone,
+    the portions of other steps to the matrix cores where they take the sizes (single tokens, which come
+    first, to their kernel), else to the vector-unit tile kernel. ``changes``: ``window``, ``chunk``, ``sink``,
+    ``r1``, ``r2`` as :func:`dli_amd.kernels.ops.attention_scored` takes them."""
+    grp = ctx.groups[cache.group]
+    nd = ctx.num_decode
+    if nd == ctx.num_entries:
+        # every entry is one row: nothing is derived from the step's lengths on the host
+        ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                             None, None, num_heads, scale, gate=gate, **changes)
+    elif ops.attention_scored_mfma_supports(head_dim, value_dim, ctx.page_size, rt.dtype):
+        if nd:
+            ops.attention_scored(q[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.q_start[:nd + 1], ctx.kv_len[:nd],
+                                 grp.block_tables[:nd], None, None, num_heads, scale,
+                                 gate=None if gate is None else gate[:nd], **changes)
+        tiles = ctx.q_tiles(ops.SCORED_MFMA_TILE_ROWS, first_entry=nd)
+        ops.attention_scored_mfma(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                                  tiles[0], tiles[1], num_heads, scale, gate=gate, **changes)
+    else:
+        tiles = ctx.q_tiles(ops.attention_generic_tile_rows(max(head_dim, value_dim)))
+        ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
+                             tiles[0], tiles[1], num_heads, scale, gate=gate, **changes)
+
+
 @register_part("mixer", "scored_attention")
 class ScoredAttention(Mixer):
     VALUE_MIX = ("none", "source", "mix")
@@ -168,23 +196,6 @@ class ScoredAttention(Mixer):
         out = self.rt.empty(n, self._o)
         g0 = self._q + self._k + self._v
         gate = proj[:, g0:g0 + self._o] if self.output_gate else None
-        changes = dict(window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2)
-        nd = ctx.num_decode
-        if nd == ctx.num_entries:
-            # every entry is one row: nothing is derived from the step's lengths on the host
-            ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
-                                 None, None, self.num_heads, self.scale, gate=gate, **changes)
-        elif ops.attention_scored_mfma_supports(self.head_dim, self.value_dim, ctx.page_size, self.rt.dtype):
-            # single tokens (they come first) to their kernel, portions to the matrix cores
-            if nd:
-                ops.attention_scored(q[:nd], cache.k_pages, cache.v_pages, out[:nd], ctx.q_start[:nd + 1], ctx.kv_len[:nd],
-                                     grp.block_tables[:nd], None, None, self.num_heads, self.scale,
-                                     gate=None if gate is None else gate[:nd], **changes)
-            tiles = ctx.q_tiles(ops.SCORED_MFMA_TILE_ROWS, first_entry=nd)
-            ops.attention_scored_mfma(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
-                                      tiles[0], tiles[1], self.num_heads, self.scale, gate=gate, **changes)
-        else:
-            tiles = ctx.q_tiles(ops.attention_generic_tile_rows(max(self.head_dim, self.value_dim)))
-            ops.attention_scored(q, cache.k_pages, cache.v_pages, out, ctx.q_start, ctx.kv_len, grp.block_tables,
-                                 tiles[0], tiles[1], self.num_heads, self.scale, gate=gate, **changes)
+        paged_scored_attention(self.rt, ctx, cache, q, out, self.num_heads, self.head_dim, self.value_dim, self.scale,
+                               gate=gate, window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2)
         return linear_f32(self.rt, out, self.w_o)
