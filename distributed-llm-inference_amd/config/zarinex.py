@@ -8,7 +8,7 @@ weights with a cache and state of its own.
 ``config.json`` keys: ``vocab``, ``width``, ``norm.eps``, ``postln_alpha`` and ``layers``: a list of
 ``{"type", "mixer": {...}, "mlp": {...} | null, "weights_of": j (optional)}``. Mixer keys by type:
 ``mamba1``: ``inner``, ``state``, ``dt_rank``, ``conv``;
-``latent_attention``: ``heads``, ``dim``, ``vdim``, ``kv_rank``, ``q_rank``, ``scale``;
+``latent_attention``: ``heads``, ``dim``, ``vdim``, ``kv_rank``, ``q_rank``, ``scale`` (absent: ``dim ** -0.5``);
 ``hgrn2``: ``heads``, ``dim``, ``vdim``.
 ``mlp``: ``{"kind": "moe", "expert": {ff}, "router": {experts, top}, "shared": {ff} | absent}``.
 """
@@ -66,7 +66,7 @@ class ZarinexLayer:
         elif kind == "latent_attention":
             sizes = {k: _positive(_need(m, k, w), f"{w}.{k}") for k in ("heads", "dim", "kv_rank", "q_rank")}
             sizes["vdim"] = _positive(m.get("vdim") or sizes["dim"], w + ".vdim")
-            sizes["scale"] = float(_need(m, "scale", w))
+            sizes["scale"] = float(m["scale"]) if m.get("scale") is not None else sizes["dim"] ** -0.5
         else:
             sizes = {k: _positive(_need(m, k, w), f"{w}.{k}") for k in ("heads", "dim")}
             sizes["vdim"] = _positive(m.get("vdim") or sizes["dim"], w + ".vdim")
