@@ -275,14 +275,35 @@ def miberax_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
             "layers": [layer(i) for i in range(layers)]}
 
 
+def zarinex_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
+    """A Zarinex of sizes that resemble a real model's layers: attention through a latent of 256 values (heads of
+    64, queries through a latent of three quarters of the width), a selective scan of twice the width with 16
+    states a channel, a low-rank step size of a sixteenth of the width and four taps, and a gated linear
+    recurrence with heads of 64, in the order attention, scan, recurrence, scan; every layer with the mixture of
+    experts that every other Miberax layer has (32 experts of an eighth of the Llama layer's hidden size, four
+    chosen, beside a shared expert of a quarter)."""
+    mixers = {
+        "latent_attention": {"heads": heads, "dim": 64, "vdim": 64, "kv_rank": 256, "q_rank": 3 * width // 4, "scale": 0.125},
+        "mamba1": {"inner": 2 * width, "state": 16, "dt_rank": width // 16, "conv": 4},
+        "hgrn2": {"heads": heads, "dim": 64, "vdim": 64},
+    }
+    mlp = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 32, "top": 4}, "shared": {"ff": ff // 4}}
+    order = ["latent_attention", "mamba1", "hgrn2", "mamba1"]
+    return {"architecture": "Zarinex", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "postln_alpha": 1.0,
+            "layers": [{"type": order[i % 4], "mixer": mixers[order[i % 4]], "mlp": mlp} for i in range(layers)]}
+
+
 DESIGN_SIZES = {  # width, heads (of 64), kv heads, feed-forward, layers, vocabulary, attention chunk
     "1024": (1024, 16, 4, 4096, 8, 32000, 1024),
     "2048": (2048, 32, 8, 8192, 8, 32000, 2048),
 }
 
 
+BESIDE = {"miberax": "makodra and ", "zarinex": "miberax and "}
+
+
 def design_compare(args):
-    """Prefill and decode throughput of Makodra beside the Llama decoder at equal width, heads,
+    """Prefill and decode throughput of a design (beside its closest earlier one) and the Llama decoder at equal width, heads,
     feed-forward, layers and vocabulary (random weights), each through the engine's own step loop."""
     import gc
 
@@ -292,8 +313,10 @@ def design_compare(args):
     for name in args.design_sizes.split(","):
         width, heads, kv_heads, ff, layers, vocab, chunk = DESIGN_SIZES[name]
         shapes = {
-            **({"miberax": miberax_shape(width, heads, kv_heads, ff, layers, vocab, chunk)} if args.design == "miberax" else {}),
-            "makodra": makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk),
+            **({"zarinex": zarinex_shape(width, heads, kv_heads, ff, layers, vocab, chunk)} if args.design == "zarinex" else {}),
+            **({"miberax": miberax_shape(width, heads, kv_heads, ff, layers, vocab, chunk)}
+               if args.design in ("miberax", "zarinex") else {}),
+            **({"makodra": makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk)} if args.design != "zarinex" else {}),
             "llama": dict(LLAMA_3_2_1B, vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
                           num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=64),
         }
@@ -408,13 +431,13 @@ def main() -> int:
                     help="prompt length of --only-prefill (the line of the default run always has 2,048)")
     ap.add_argument("--portion", type=int, default=None,
                     help="with --only-prefill: the prompt runs in steps of at most this many tokens")
-    ap.add_argument("--design", default=None, choices=["makodra", "miberax"],
+    ap.add_argument("--design", default=None, choices=["makodra", "miberax", "zarinex"],
                     help="instead of the default run: prefill (2,048 and 8,192 tokens) and decode (batch 1, 8, 64 at "
                          "--context) of this design beside the Llama decoder at equal sizes, random weights")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design, of " + ", ".join(DESIGN_SIZES))
     ap.add_argument("--design-phases", default="prefill2048,prefill8192,decode_b1,decode_b8,decode_b64",
                     help="with --design: which of these measurements to make")
-    ap.add_argument("--design-only", default=None, choices=["makodra", "miberax", "llama"],
+    ap.add_argument("--design-only", default=None, choices=["makodra", "miberax", "zarinex", "llama"],
                     help="with --design: measure this one of the pair alone (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -438,7 +461,7 @@ def main() -> int:
     itemsize = 2 if short == "bf16" else 4
     if args.design:
         print(json.dumps({
-            "metric": f"{args.design} beside {'makodra and ' if args.design == 'miberax' else ''}llama at equal sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
+            "metric": f"{args.design} beside {BESIDE.get(args.design, '')}llama at equal sizes: prefill and decode tok/s", "unit": "tok/s", "n_gpus": 1,
             "dtype": short, "data": "synthetic: random token ids, random-init weights N(0, 0.02)",
             "config": {"context": args.context, "kv_block_size": args.block_size, "sizes": {
                 n: dict(zip(("width", "heads_of_64", "kv_heads", "ff", "layers", "vocab", "chunk"), DESIGN_SIZES[n]))

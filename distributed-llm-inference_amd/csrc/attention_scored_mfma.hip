@@ -13,8 +13,9 @@
 // r1 log2(1 + r2 d) in that domain (one v_log_f32). P is rounded to bfloat16 for the second product
 // while the running sum keeps the unrounded values, as in the other matrix-core attention.
 //
-// Needs head_dim and value_dim of 16 to 96 in steps of 16, or 128, and page_size % 4 == 0; other
-// shapes, and the 32-bit runtime, take the vector-unit kernel.
+// Needs head_dim and value_dim of 16 to 96 in steps of 16, or 128 (or, where values are as long as keys,
+// as when a cached latent is both, any multiple of 16 up to 256), and page_size % 4 == 0; other shapes,
+// and the 32-bit runtime, take the vector-unit kernel.
 #include "common.h"
 
 typedef short short4s __attribute__((ext_vector_type(4)));
@@ -153,8 +154,8 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
 // Whether the matrix-core kernel takes these sizes (tiles of 64 queries).
 extern "C" int dli_attention_scored_mfma_supports(int head_dim, int value_dim, int page_size) {
   const int dt = head_dim / 16, vt = value_dim / 16;
-  return head_dim > 0 && value_dim > 0 && head_dim % 16 == 0 && value_dim % 16 == 0 && (dt <= 6 || dt == 8) &&
-         (vt <= 6 || vt == 8) && page_size > 0 && page_size % 4 == 0;
+  return head_dim > 0 && value_dim > 0 && head_dim % 16 == 0 && value_dim % 16 == 0 &&
+         (((dt <= 6 || dt == 8) && (vt <= 6 || vt == 8)) || (dt == vt && dt <= 16)) && page_size > 0 && page_size % 4 == 0;
 }
 
 template <int DT>
@@ -166,6 +167,13 @@ static int launch_scored_mfma(const ScoredArgs& a, int tiles, int value_dim, hip
     default: return DLI_ERR_ARGUMENT;
   }
 #undef VCASE
+  return dli_launch_status();
+}
+
+// Values as long as keys, of the sizes that the cases above leave out.
+template <int DT>
+static int launch_scored_mfma_square(const ScoredArgs& a, int tiles, hipStream_t stream) {
+  attention_scored_mfma_kernel<DT, DT><<<dim3(tiles, a.q_heads), 256, 0, stream>>>(a);
   return dli_launch_status();
 }
 
@@ -196,6 +204,15 @@ extern "C" int dli_attention_scored_mfma(const void* q, int64_t q_stride, const 
     case 5: return launch_scored_mfma<5>(a, tiles, value_dim, stream);
     case 6: return launch_scored_mfma<6>(a, tiles, value_dim, stream);
     case 8: return launch_scored_mfma<8>(a, tiles, value_dim, stream);
+    case 7: return launch_scored_mfma_square<7>(a, tiles, stream);
+    case 9: return launch_scored_mfma_square<9>(a, tiles, stream);
+    case 10: return launch_scored_mfma_square<10>(a, tiles, stream);
+    case 11: return launch_scored_mfma_square<11>(a, tiles, stream);
+    case 12: return launch_scored_mfma_square<12>(a, tiles, stream);
+    case 13: return launch_scored_mfma_square<13>(a, tiles, stream);
+    case 14: return launch_scored_mfma_square<14>(a, tiles, stream);
+    case 15: return launch_scored_mfma_square<15>(a, tiles, stream);
+    case 16: return launch_scored_mfma_square<16>(a, tiles, stream);
     default: return DLI_ERR_ARGUMENT;
   }
 }

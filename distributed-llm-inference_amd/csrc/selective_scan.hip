@@ -11,7 +11,8 @@
 //
 // Sixteen lanes (a DPP row) share a channel: lane `part` keeps the states n = part + 16 j, j < NPER, in
 // registers (so the 16 lanes read B and C as one run), and a token's sum over n meets in four DPP
-// swaps. A wave takes four channels, a workgroup sixteen. N up to 256.
+// swaps. A wave takes four channels, a workgroup sixteen. N up to 256. A few tokens' operands are held in
+// registers while the next few are in flight.
 #include "common.h"
 
 struct SsmArgs {
@@ -64,24 +65,57 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SsmArgs p) {
     s[j] = (fresh || !valid[j]) ? 0.f : old;
   }
   const float dc = p.d != nullptr ? p.d[c] : 0.f;
-#pragma unroll 2
-  for (int t = 0; t < n_rows; ++t) {
-    const int64_t row = row0 + t;
-    const float dtv = dt[row * p.dt_stride + c], xv = x[row * p.x_stride + c];
-    const float dx = dtv * xv;
-    float acc = 0.f;
+  // TB tokens' operands are asked for while the TB before them are computed: the chain over tokens is one
+  // multiply-add a state, and nothing on it waits for memory. The decay is exp2 of a product with log2(e)
+  // folded into A.
+  constexpr int TB = NPER <= 2 ? 8 : NPER <= 4 ? 4 : NPER <= 8 ? 2 : 1;
+  constexpr float LOG2E = 1.4426950408889634f;
 #pragma unroll
-    for (int j = 0; j < NPER; ++j) {
-      const float b = bc[row * p.bc_stride + p.b_off + at[j]], cc = bc[row * p.bc_stride + p.c_off + at[j]];
-      s[j] = valid[j] ? fmaf(expf(dtv * a[j]), s[j], dx * b) : 0.f;
-      acc = fmaf(s[j], cc, acc);
+  for (int j = 0; j < NPER; ++j) a[j] *= LOG2E;
+  float dt_n[TB], x_n[TB], z_n[TB], b_n[TB][NPER], c_n[TB][NPER];
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const int64_t row = row0 + min(t0 + i, n_rows - 1);
+      dt_n[i] = dt[row * p.dt_stride + c];
+      x_n[i] = x[row * p.x_stride + c];
+      z_n[i] = z != nullptr ? z[row * p.z_stride + c] : 0.f;
+#pragma unroll
+      for (int j = 0; j < NPER; ++j) {
+        b_n[i][j] = bc[row * p.bc_stride + p.b_off + at[j]];
+        c_n[i][j] = bc[row * p.bc_stride + p.c_off + at[j]];
+      }
     }
-    float y = fmaf(dc, xv, ssm_row_sum(acc));
-    if (z != nullptr) {
-      const float g = z[row * p.z_stride + c];
-      y *= g / (1.f + expf(-g));
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < n_rows; t0 += TB) {
+    float dt_c[TB], x_c[TB], z_c[TB], b_c[TB][NPER], c_c[TB][NPER];
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      dt_c[i] = dt_n[i]; x_c[i] = x_n[i]; z_c[i] = z_n[i];
+#pragma unroll
+      for (int j = 0; j < NPER; ++j) { b_c[i][j] = b_n[i][j]; c_c[i][j] = c_n[i][j]; }
     }
-    if (part == 0 && live) out[row * p.out_stride + c] = from_f32<T>(y);
+    if (t0 + TB < n_rows) fetch(t0 + TB);
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      if (t0 + i < n_rows) {                 // (the same for every lane of the workgroup)
+        const float dtv = dt_c[i], xv = x_c[i];
+        const float dx = dtv * xv;
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < NPER; ++j) {
+          s[j] = valid[j] ? fmaf(__builtin_amdgcn_exp2f(dtv * a[j]), s[j], dx * b_c[i][j]) : 0.f;
+          acc = fmaf(s[j], c_c[i][j], acc);
+        }
+        float y = fmaf(dc, xv, ssm_row_sum(acc));
+        if (z != nullptr) {
+          const float g = z_c[i];
+          y *= g / (1.f + __expf(-g));
+        }
+        if (part == 0 && live) out[(row0 + t0 + i) * p.out_stride + c] = from_f32<T>(y);
+      }
+    }
   }
   if (live)
 #pragma unroll
