@@ -230,7 +230,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
     const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k_pages, const T* __restrict__ v_pages,
     T* __restrict__ out, int64_t out_stride, const int* __restrict__ kv_len, const int* __restrict__ block_tables,
     int table_stride, int q_heads, int kv_heads, int head_dim, int page_size, float scale, int window,
-    ScoreChanges sc) {
+    ScoreChanges sc, float* __restrict__ parts, int splits) {
   constexpr int PN = Pack16<T>::N;
   typedef typename Pack16<T>::type P16;
   extern __shared__ float lds[];
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
   float* ps = qs + GQ * head_dim;                // [waves][GQ][64]
   float* ms = ps + waves * GQ * 64;              // [waves][GQ] reference points, then [waves][GQ] sums
   float* accs = ms + 2 * waves * GQ;             // [waves][GQ][VC * 64]
-  const int entry = blockIdx.x, kvh = blockIdx.y;
+  const int entry = blockIdx.x / splits, split = blockIdx.x % splits, kvh = blockIdx.y;
   const int group = q_heads / kv_heads;
   const int h0 = kvh * group + blockIdx.z * GQ;                  // first query head of this workgroup
   const int nh = min(GQ, kvh * group + group - h0);              // heads that exist
@@ -257,8 +257,8 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
   for (int h = 0; h < GQ; ++h) {
     r1[h] = sc.r1 != nullptr && h < nh ? sc.r1[h0 + h] : 0.f;
     r2[h] = sc.r1 != nullptr && h < nh ? sc.r2[h0 + h] : 0.f;
-    m_run[h] = sc.sink && wave == 0 ? 0.f : -INFINITY;           // the sink is counted once, by wave 0
-    l_run[h] = sc.sink && wave == 0 && lane == 0 ? 1.f : 0.f;    // (sums are kept lane by lane until the end)
+    m_run[h] = sc.sink && wave == 0 && split == 0 ? 0.f : -INFINITY;           // the sink is counted once, by wave 0
+    l_run[h] = sc.sink && wave == 0 && split == 0 && lane == 0 ? 1.f : 0.f;    // (sums are kept lane by lane until the end)
 #pragma unroll
     for (int c = 0; c < VC; ++c) acc[h][c] = 0.f;
   }
@@ -268,7 +268,8 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
   __syncthreads();
 
   const bool k_packs = head_dim % PN == 0, v_packs = page_size % PN == 0;
-  for (int j0 = j_begin / 64 * 64 + wave * 64; j0 <= pos; j0 += 64 * waves) {
+  // blocks of 64 keys go round the waves of the `splits` workgroups that share this (entry, heads)
+  for (int j0 = j_begin / 64 * 64 + (split * waves + wave) * 64; j0 <= pos; j0 += 64 * waves * splits) {
     const int j = j0 + lane;
     const bool seen = j >= j_begin && j <= pos;
     // the page of this lane's key, for its own row of K and, handed round, for the rows of V (a key
@@ -401,9 +402,46 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
         o += accs[((w * GQ + h) * VC + col / 64) * 64 + col % 64] * f;
       }
     }
+    if (splits > 1) {
+      // this workgroup's share: the sum as it is, with its reference point and denominator behind it
+      float* part = parts + (((int64_t)entry * q_heads + h0 + h) * splits + split) * (value_dim + 2);
+      part[col] = o;
+      if (col == 0) {
+        part[value_dim] = m;
+        part[value_dim + 1] = l;
+      }
+      continue;
+    }
     float y = l > 0.f ? o / l : 0.f;
     const int64_t at = (int64_t)(h0 + h) * value_dim + col;
     if (sc.gate != nullptr) y *= 1.f / (1.f + expf(-sc.gate[(int64_t)entry * sc.gate_stride + at]));
+    out[(int64_t)entry * out_stride + at] = from_f32<T>(y);
+  }
+}
+
+// The shares of the workgroups that split an entry's keys meet: parts [entries][q_heads][splits][value_dim + 2].
+// One workgroup an (entry, head), a thread a value column; sums in the order of the splits.
+template <typename T>
+__global__ void attention_scored_merge_kernel(const float* __restrict__ parts, int splits, int q_heads, int value_dim,
+                                              const float* __restrict__ gate, int64_t gate_stride, T* __restrict__ out,
+                                              int64_t out_stride) {
+  const int entry = blockIdx.x, head = blockIdx.y;
+  const float* base = parts + ((int64_t)entry * q_heads + head) * splits * (value_dim + 2);
+  float m = -INFINITY;
+  for (int s = 0; s < splits; ++s) m = fmaxf(m, base[s * (value_dim + 2) + value_dim]);
+  for (int col = threadIdx.x; col < value_dim; col += blockDim.x) {
+    float l = 0.f, o = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = base[s * (value_dim + 2) + value_dim];
+      if (ms > -INFINITY) {
+        const float f = expf(ms - m);
+        l += base[s * (value_dim + 2) + value_dim + 1] * f;
+        o += base[s * (value_dim + 2) + col] * f;
+      }
+    }
+    float y = l > 0.f ? o / l : 0.f;
+    const int64_t at = (int64_t)head * value_dim + col;
+    if (gate != nullptr) y *= 1.f / (1.f + expf(-gate[(int64_t)entry * gate_stride + at]));
     out[(int64_t)entry * out_stride + at] = from_f32<T>(y);
   }
 }
@@ -412,9 +450,11 @@ template <typename T, int GQ>
 static int launch_scored_decode(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages, void* out,
                                 int64_t out_stride, const int* kv_len, const int* block_tables, int table_stride,
                                 int entries, int q_heads, int kv_heads, int head_dim, int page_size, float scale,
-                                int window, ScoreChanges sc, hipStream_t stream) {
+                                int window, ScoreChanges sc, float* parts, int splits, hipStream_t stream) {
   const int group = q_heads / kv_heads, vc = (sc.value_dim + 63) / 64;
-  const dim3 grid(entries, kv_heads, (group + GQ - 1) / GQ);
+  if (parts == nullptr || splits < 1) splits = 1;
+  if ((int64_t)entries * splits > 0x7fffffff) return DLI_ERR_ARGUMENT;
+  const dim3 grid(entries * splits, kv_heads, (group + GQ - 1) / GQ);
   // eight waves where their states fit 64 KB of LDS, else four: the chain of a wave's
   // blocks (table entry, key rows, value rows, each a trip to memory) is as long as its blocks
 #define DECODE_LAUNCH(VC)                                                                                   \
@@ -427,10 +467,17 @@ static int launch_scored_decode(const void* q, int64_t q_stride, const void* k_p
     }                                                                                                       \
     attention_scored_decode_kernel<T, GQ, VC><<<grid, 64 * waves, bytes, stream>>>(                         \
         (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, (T*)out, out_stride, kv_len,           \
-        block_tables, table_stride, q_heads, kv_heads, head_dim, page_size, scale, window, sc);             \
+        block_tables, table_stride, q_heads, kv_heads, head_dim, page_size, scale, window, sc, parts, splits); \
   }
   if (vc <= 1) DECODE_LAUNCH(1) else if (vc == 2) DECODE_LAUNCH(2) else DECODE_LAUNCH(4)
 #undef DECODE_LAUNCH
+  if (splits > 1) {
+    const int status = dli_launch_status();
+    if (status != DLI_OK) return status;
+    attention_scored_merge_kernel<T><<<dim3(entries, q_heads), sc.value_dim <= 64 ? 64 : sc.value_dim <= 128 ? 128 : 256, 0,
+                                       stream>>>(parts, splits, q_heads, sc.value_dim, sc.gate, sc.gate_stride, (T*)out,
+                                                 out_stride);
+  }
   return dli_launch_status();
 }
 
@@ -443,14 +490,14 @@ extern "C" int dli_attention_generic_tile_rows(int head_dim) {
 
 // The attention with every change to the scores as a parameter (see the head of this file).
 // chunk 0, sink 0, r1 = r2 = gate = nullptr and value_dim == head_dim: the plain attention.
-extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void* k_pages,
-                                    const void* v_pages, void* out, int64_t out_stride,
-                                    const int* q_start, const int* kv_len, const int* block_tables,
-                                    int table_stride, const int* tile_entry, const int* tile_q0,
-                                    int tiles, int q_heads, int kv_heads, int head_dim, int value_dim,
-                                    int page_size, float scale, int window, int chunk, int sink,
-                                    const float* r1, const float* r2, const float* gate,
-                                    int64_t gate_stride, int is_bf16, hipStream_t stream) {
+static int attention_scored(const void* q, int64_t q_stride, const void* k_pages,
+                            const void* v_pages, void* out, int64_t out_stride,
+                            const int* q_start, const int* kv_len, const int* block_tables,
+                            int table_stride, const int* tile_entry, const int* tile_q0,
+                            int tiles, int q_heads, int kv_heads, int head_dim, int value_dim,
+                            int page_size, float scale, int window, int chunk, int sink,
+                            const float* r1, const float* r2, const float* gate,
+                            int64_t gate_stride, float* parts, int splits, int is_bf16, hipStream_t stream) {
   if (tiles <= 0) return DLI_OK;
   const int dmax = head_dim > value_dim ? head_dim : value_dim;
   if (head_dim <= 0 || value_dim <= 0 || dmax > 256 || q_heads <= 0 || kv_heads <= 0 ||
@@ -464,7 +511,7 @@ extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void*
     const int group = q_heads / kv_heads;
 #define DECODE_ARGS                                                                                      \
   q, q_stride, k_pages, v_pages, out, out_stride, kv_len, block_tables, table_stride, tiles, q_heads,   \
-      kv_heads, head_dim, page_size, scale, window, sc, stream
+      kv_heads, head_dim, page_size, scale, window, sc, parts, splits, stream
     if (is_bf16) {
       if (group == 1) return launch_scored_decode<bf16_t, 1>(DECODE_ARGS);
       if (group <= 4) return launch_scored_decode<bf16_t, 4>(DECODE_ARGS);
@@ -489,6 +536,45 @@ extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void*
 #undef GENERIC_ARGS
 }
 
+extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void* k_pages,
+                                    const void* v_pages, void* out, int64_t out_stride,
+                                    const int* q_start, const int* kv_len, const int* block_tables,
+                                    int table_stride, const int* tile_entry, const int* tile_q0,
+                                    int tiles, int q_heads, int kv_heads, int head_dim, int value_dim,
+                                    int page_size, float scale, int window, int chunk, int sink,
+                                    const float* r1, const float* r2, const float* gate,
+                                    int64_t gate_stride, int is_bf16, hipStream_t stream) {
+  return attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len, block_tables, table_stride,
+                          tile_entry, tile_q0, tiles, q_heads, kv_heads, head_dim, value_dim, page_size, scale, window,
+                          chunk, sink, r1, r2, gate, gate_stride, nullptr, 1, is_bf16, stream);
+}
+
+// How many workgroups share the keys of an (entry, group of query heads) in a step of single tokens. It
+// depends on the heads alone, never on the step, so that a row's sums are made in one order whatever
+// else is in the batch: few (kv head, head group) pairs an entry leave the chip idle unless the keys
+// are cut.
+extern "C" int dli_attention_scored_splits(int q_heads, int kv_heads) {
+  if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return 1;
+  const int group = q_heads / kv_heads, gq = group == 1 ? 1 : group <= 4 ? 4 : 8;
+  const int per_entry = kv_heads * ((group + gq - 1) / gq);
+  const int splits = 32 / per_entry;
+  return splits < 1 ? 1 : splits > 16 ? 16 : splits;
+}
+
+// A step of single tokens (every entry one row) with each entry's keys cut over `splits` workgroups:
+// parts is float [entries * q_heads * splits * (value_dim + 2)] of scratch.
+extern "C" int dli_attention_scored_single(const void* q, int64_t q_stride, const void* k_pages, const void* v_pages,
+                                           void* out, int64_t out_stride, const int* kv_len, const int* block_tables,
+                                           int table_stride, int entries, int q_heads, int kv_heads, int head_dim,
+                                           int value_dim, int page_size, float scale, int window, int chunk, int sink,
+                                           const float* r1, const float* r2, const float* gate, int64_t gate_stride,
+                                           float* parts, int splits, int is_bf16, hipStream_t stream) {
+  if (splits < 1 || splits > 64 || (splits > 1 && parts == nullptr)) return DLI_ERR_ARGUMENT;
+  return attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, nullptr, kv_len, block_tables, table_stride,
+                          nullptr, nullptr, entries, q_heads, kv_heads, head_dim, value_dim, page_size, scale, window,
+                          chunk, sink, r1, r2, gate, gate_stride, parts, splits, is_bf16, stream);
+}
+
 extern "C" int dli_attention_generic(const void* q, int64_t q_stride, const void* k_pages,
                                      const void* v_pages, void* out, int64_t out_stride,
                                      const int* q_start, const int* kv_len, const int* block_tables,
@@ -496,8 +582,8 @@ extern "C" int dli_attention_generic(const void* q, int64_t q_stride, const void
                                      int tiles, int q_heads, int kv_heads, int head_dim, int page_size,
                                      float scale, int window, int is_bf16, hipStream_t stream) {
   if (head_dim % 16 != 0 || tile_entry == nullptr) return tiles <= 0 ? DLI_OK : DLI_ERR_ARGUMENT;
-  return dli_attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len,
-                              block_tables, table_stride, tile_entry, tile_q0, tiles, q_heads,
-                              kv_heads, head_dim, head_dim, page_size, scale, window, 0, 0, nullptr,
-                              nullptr, nullptr, 0, is_bf16, stream);
+  return attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len,
+                          block_tables, table_stride, tile_entry, tile_q0, tiles, q_heads,
+                          kv_heads, head_dim, head_dim, page_size, scale, window, 0, 0, nullptr,
+                          nullptr, nullptr, 0, nullptr, 1, is_bf16, stream);
 }

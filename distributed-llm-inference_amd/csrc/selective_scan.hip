@@ -97,24 +97,34 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SsmArgs p) {
       for (int j = 0; j < NPER; ++j) { b_c[i][j] = b_n[i][j]; c_c[i][j] = c_n[i][j]; }
     }
     if (t0 + TB < n_rows) fetch(t0 + TB);
+    // everything of a token that is not on the chain over tokens is made for all TB at once: decays,
+    // inputs and the gate's factor; then the chain, then the sums over the sixteen lanes
+    float decay[TB][NPER], gate[TB], y[TB];
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
-      if (t0 + i < n_rows) {                 // (the same for every lane of the workgroup)
-        const float dtv = dt_c[i], xv = x_c[i];
-        const float dx = dtv * xv;
-        float acc = 0.f;
 #pragma unroll
-        for (int j = 0; j < NPER; ++j) {
-          s[j] = valid[j] ? fmaf(__builtin_amdgcn_exp2f(dtv * a[j]), s[j], dx * b_c[i][j]) : 0.f;
-          acc = fmaf(s[j], c_c[i][j], acc);
-        }
-        float y = fmaf(dc, xv, ssm_row_sum(acc));
-        if (z != nullptr) {
-          const float g = z_c[i];
-          y *= g / (1.f + __expf(-g));
-        }
-        if (part == 0 && live) out[(row0 + t0 + i) * p.out_stride + c] = from_f32<T>(y);
+      for (int j = 0; j < NPER; ++j) decay[i][j] = __builtin_amdgcn_exp2f(dt_c[i] * a[j]);
+      const float g = z_c[i];
+      gate[i] = z != nullptr ? g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) : 1.f;
+    }
+    const int full = min(TB, n_rows - t0);       // (the same for every lane of the workgroup)
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const float dx = dt_c[i] * x_c[i];
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < NPER; ++j) {
+        // rows past the step's last repeat it and change nothing
+        const float next = valid[j] ? fmaf(decay[i][j], s[j], dx * b_c[i][j]) : 0.f;
+        s[j] = i < full ? next : s[j];
+        acc = fmaf(next, c_c[i][j], acc);
       }
+      y[i] = acc;
+    }
+#pragma unroll
+    for (int i = 0; i < TB; ++i) {
+      const float v = fmaf(dc, x_c[i], ssm_row_sum(y[i])) * gate[i];
+      if (part == 0 && live && i < full) out[(row0 + t0 + i) * p.out_stride + c] = from_f32<T>(v);
     }
   }
   if (live)

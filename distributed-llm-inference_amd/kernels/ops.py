@@ -100,6 +100,10 @@ _SIGNATURES = {
     "dli_attention_scored": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
                              _c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
+    "dli_attention_scored_splits": [_c_int, _c_int],
+    "dli_attention_scored_single": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                                    _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64,
+                                    _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_scored_mfma_supports": [_c_int, _c_int, _c_int],
     "dli_attention_scored_mfma": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
@@ -1606,6 +1610,18 @@ def attention_scored(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
         _f32_rows(gate, "gate")
         _require(gate.shape == out.shape, "gate differs from out in shape")
         gate_stride = gate.stride(0)
+    if tile_entry is None:
+        # few (kv head, group of query heads) pairs an entry: an entry's keys are cut over several workgroups
+        # (a number that the heads alone decide), whose shares a second kernel adds up
+        splits = int(library().dli_attention_scored_splits(q_heads, kv_heads))
+        if splits > 1:
+            parts = torch.empty(entries * q_heads * splits * (value_dim + 2), device=q.device, dtype=torch.float32)
+            _check(library().dli_attention_scored_single(
+                _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(kv_len),
+                _ptr(block_tables), block_tables.stride(0), entries, q_heads, kv_heads, head_dim, value_dim, page_size,
+                float(scale), int(window), int(chunk), int(bool(sink)), _ptr(r1), _ptr(r2), _ptr(gate), gate_stride,
+                _ptr(parts), splits, _is_bf16(dtype), _stream()), "attention_scored_single")
+            return
     _check(library().dli_attention_scored(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
         _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tiles, q_heads, kv_heads,
