@@ -549,16 +549,16 @@ extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void*
                           chunk, sink, r1, r2, gate, gate_stride, nullptr, 1, is_bf16, stream);
 }
 
-// How many workgroups share the keys of an (entry, group of query heads) in a step of single tokens. It
-// depends on the heads alone, never on the step, so that a row's sums are made in one order whatever
-// else is in the batch: few (kv head, head group) pairs an entry leave the chip idle unless the keys
-// are cut.
-extern "C" int dli_attention_scored_splits(int q_heads, int kv_heads) {
-  if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0) return 1;
+// How many workgroups share the keys of an (entry, group of query heads) in a step of single tokens: as
+// many as bring the launch to about two workgroups a compute unit, sixteen at most. It depends on the
+// heads and the number of entries, never on their lengths. A step of many entries fills the chip by
+// itself and is not cut (cutting it costs more than it gains).
+extern "C" int dli_attention_scored_splits(int q_heads, int kv_heads, int entries) {
+  if (q_heads <= 0 || kv_heads <= 0 || q_heads % kv_heads != 0 || entries <= 0) return 1;
   const int group = q_heads / kv_heads, gq = group == 1 ? 1 : group <= 4 ? 4 : 8;
-  const int per_entry = kv_heads * ((group + gq - 1) / gq);
-  const int splits = 32 / per_entry;
-  return splits < 1 ? 1 : splits > 16 ? 16 : splits;
+  const int64_t workgroups = (int64_t)entries * kv_heads * ((group + gq - 1) / gq);
+  const int64_t splits = 512 / workgroups;
+  return splits < 1 ? 1 : splits > 16 ? 16 : (int)splits;
 }
 
 // A step of single tokens (every entry one row) with each entry's keys cut over `splits` workgroups:

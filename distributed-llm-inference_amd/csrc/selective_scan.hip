@@ -65,67 +65,73 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SsmArgs p) {
     s[j] = (fresh || !valid[j]) ? 0.f : old;
   }
   const float dc = p.d != nullptr ? p.d[c] : 0.f;
-  // TB tokens' operands are asked for while the TB before them are computed: the chain over tokens is one
-  // multiply-add a state, and nothing on it waits for memory. The decay is exp2 of a product with log2(e)
-  // folded into A.
+  // Tokens go in blocks of TB whose operands are asked for two blocks ahead: the chain over tokens is
+  // one multiply-add a state, and nothing on it waits for memory. The decay is exp2 of a product with
+  // log2(e) folded into A.
   constexpr int TB = NPER <= 2 ? 8 : NPER <= 4 ? 4 : NPER <= 8 ? 2 : 1;
   constexpr float LOG2E = 1.4426950408889634f;
 #pragma unroll
   for (int j = 0; j < NPER; ++j) a[j] *= LOG2E;
-  float dt_n[TB], x_n[TB], z_n[TB], b_n[TB][NPER], c_n[TB][NPER];
-  auto fetch = [&](int t0) {
+  struct Block { float dt[TB], x[TB], z[TB], b[TB][NPER], c[TB][NPER]; };
+  auto fetch = [&](Block& k, int t0) {        // rows past the step's last repeat it
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
       const int64_t row = row0 + min(t0 + i, n_rows - 1);
-      dt_n[i] = dt[row * p.dt_stride + c];
-      x_n[i] = x[row * p.x_stride + c];
-      z_n[i] = z != nullptr ? z[row * p.z_stride + c] : 0.f;
+      k.dt[i] = dt[row * p.dt_stride + c];
+      k.x[i] = x[row * p.x_stride + c];
+      k.z[i] = z != nullptr ? z[row * p.z_stride + c] : 0.f;
 #pragma unroll
       for (int j = 0; j < NPER; ++j) {
-        b_n[i][j] = bc[row * p.bc_stride + p.b_off + at[j]];
-        c_n[i][j] = bc[row * p.bc_stride + p.c_off + at[j]];
+        k.b[i][j] = bc[row * p.bc_stride + p.b_off + at[j]];
+        k.c[i][j] = bc[row * p.bc_stride + p.c_off + at[j]];
       }
     }
   };
-  fetch(0);
-  for (int t0 = 0; t0 < n_rows; t0 += TB) {
-    float dt_c[TB], x_c[TB], z_c[TB], b_c[TB][NPER], c_c[TB][NPER];
-#pragma unroll
-    for (int i = 0; i < TB; ++i) {
-      dt_c[i] = dt_n[i]; x_c[i] = x_n[i]; z_c[i] = z_n[i];
-#pragma unroll
-      for (int j = 0; j < NPER; ++j) { b_c[i][j] = b_n[i][j]; c_c[i][j] = c_n[i][j]; }
-    }
-    if (t0 + TB < n_rows) fetch(t0 + TB);
+  auto compute = [&](const Block& k, int t0) {
     // everything of a token that is not on the chain over tokens is made for all TB at once: decays,
     // inputs and the gate's factor; then the chain, then the sums over the sixteen lanes
     float decay[TB][NPER], gate[TB], y[TB];
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
 #pragma unroll
-      for (int j = 0; j < NPER; ++j) decay[i][j] = __builtin_amdgcn_exp2f(dt_c[i] * a[j]);
-      const float g = z_c[i];
+      for (int j = 0; j < NPER; ++j) decay[i][j] = __builtin_amdgcn_exp2f(k.dt[i] * a[j]);
+      const float g = k.z[i];
       gate[i] = z != nullptr ? g * __builtin_amdgcn_rcpf(1.f + __expf(-g)) : 1.f;
     }
     const int full = min(TB, n_rows - t0);       // (the same for every lane of the workgroup)
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
-      const float dx = dt_c[i] * x_c[i];
+      const float dx = k.dt[i] * k.x[i];
       float acc = 0.f;
 #pragma unroll
       for (int j = 0; j < NPER; ++j) {
-        // rows past the step's last repeat it and change nothing
-        const float next = valid[j] ? fmaf(decay[i][j], s[j], dx * b_c[i][j]) : 0.f;
+        // rows past the step's last change nothing
+        const float next = valid[j] ? fmaf(decay[i][j], s[j], dx * k.b[i][j]) : 0.f;
         s[j] = i < full ? next : s[j];
-        acc = fmaf(next, c_c[i][j], acc);
+        acc = fmaf(next, k.c[i][j], acc);
       }
       y[i] = acc;
     }
 #pragma unroll
     for (int i = 0; i < TB; ++i) {
-      const float v = fmaf(dc, x_c[i], ssm_row_sum(y[i])) * gate[i];
+      const float v = fmaf(dc, k.x[i], ssm_row_sum(y[i])) * gate[i];
       if (part == 0 && live && i < full) out[(row0 + t0 + i) * p.out_stride + c] = from_f32<T>(v);
     }
+  };
+  // three blocks of registers go round: while one is computed the next two are in flight, so a block's
+  // trip to memory has two blocks' arithmetic to hide behind
+  Block k0, k1, k2;
+  fetch(k0, 0);
+  fetch(k1, TB);
+  for (int t0 = 0; t0 < n_rows; t0 += 3 * TB) {
+    fetch(k2, t0 + 2 * TB);
+    compute(k0, t0);
+    if (t0 + TB >= n_rows) break;
+    fetch(k0, t0 + 3 * TB);
+    compute(k1, t0 + TB);
+    if (t0 + 2 * TB >= n_rows) break;
+    fetch(k1, t0 + 4 * TB);
+    compute(k2, t0 + 2 * TB);
   }
   if (live)
 #pragma unroll

@@ -100,7 +100,7 @@ _SIGNATURES = {
     "dli_attention_scored": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
                              _c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
-    "dli_attention_scored_splits": [_c_int, _c_int],
+    "dli_attention_scored_splits": [_c_int, _c_int, _c_int],
     "dli_attention_scored_single": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                                     _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64,
                                     _c_ptr, _c_int, _c_int, _c_ptr],
@@ -1612,8 +1612,8 @@ def attention_scored(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
         gate_stride = gate.stride(0)
     if tile_entry is None:
         # few (kv head, group of query heads) pairs an entry: an entry's keys are cut over several workgroups
-        # (a number that the heads alone decide), whose shares a second kernel adds up
-        splits = int(library().dli_attention_scored_splits(q_heads, kv_heads))
+        # (a number that the heads and the number of entries decide), whose shares a second kernel adds up
+        splits = int(library().dli_attention_scored_splits(q_heads, kv_heads, entries))
         if splits > 1:
             parts = torch.empty(entries * q_heads * splits * (value_dim + 2), device=q.device, dtype=torch.float32)
             _check(library().dli_attention_scored_single(
