@@ -37,7 +37,8 @@ __device__ __forceinline__ float ssm_row_sum(float x) {
   return x;
 }
 
-template <typename T, int NPER>
+// SINGLE: every entry is one row (a step of single tokens): blocks of one token.
+template <typename T, int NPER, bool SINGLE>
 __global__ __launch_bounds__(256) void selective_scan_kernel(SsmArgs p) {
   const int entry = blockIdx.x;
   const int ch = blockIdx.y * 16 + threadIdx.x / 16, part = threadIdx.x % 16;
@@ -68,7 +69,7 @@ __global__ __launch_bounds__(256) void selective_scan_kernel(SsmArgs p) {
   // Tokens go in blocks of TB whose operands are asked for two blocks ahead: the chain over tokens is
   // one multiply-add a state, and nothing on it waits for memory. The decay is exp2 of a product with
   // log2(e) folded into A.
-  constexpr int TB = NPER <= 2 ? 8 : NPER <= 4 ? 4 : NPER <= 8 ? 2 : 1;
+  constexpr int TB = SINGLE ? 1 : NPER <= 2 ? 8 : NPER <= 4 ? 4 : NPER <= 8 ? 2 : 1;
   constexpr float LOG2E = 1.4426950408889634f;
 #pragma unroll
   for (int j = 0; j < NPER; ++j) a[j] *= LOG2E;
@@ -163,8 +164,11 @@ int dli_selective_scan(const float* x, int64_t x_stride, const float* dt, int64_
   const int per = (n + 15) / 16;
 #define SSM_LAUNCH(NPER)                                                                \
   {                                                                                     \
-    if (out_is_bf16) selective_scan_kernel<bf16_t, NPER><<<grid, 256, 0, stream>>>(p);  \
-    else selective_scan_kernel<float, NPER><<<grid, 256, 0, stream>>>(p);               \
+    if (rows == entries) {                                                              \
+      if (out_is_bf16) selective_scan_kernel<bf16_t, NPER, true><<<grid, 256, 0, stream>>>(p);   \
+      else selective_scan_kernel<float, NPER, true><<<grid, 256, 0, stream>>>(p);       \
+    } else if (out_is_bf16) selective_scan_kernel<bf16_t, NPER, false><<<grid, 256, 0, stream>>>(p); \
+    else selective_scan_kernel<float, NPER, false><<<grid, 256, 0, stream>>>(p);        \
   }
   if (per <= 1) SSM_LAUNCH(1) else if (per <= 2) SSM_LAUNCH(2) else if (per <= 4) SSM_LAUNCH(4)
   else if (per <= 8) SSM_LAUNCH(8) else SSM_LAUNCH(16)
