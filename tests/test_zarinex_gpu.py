@@ -310,7 +310,7 @@ def test_a_key_far_back_is_found_through_the_latent(ops, dtype, H, d, dv, r, q_r
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("n,width,ff,experts,top", [(70, 64, 32, 6, 3), (3, 40, 24, 4, 1), (1, 96, 100, 9, 4), (130, 128, 96, 12, 2),
-                                                    (5, 48, 20, 3, 3)])
+                                                    (5, 48, 20, 3, 3), (9, 64, 32, 100, 5)])
 def test_router_with_a_bias_and_plain_silu_experts(ops, dtype, n, width, ff, experts, top):
     g = torch.Generator().manual_seed(n * 10 + experts)
     rnd = lambda *s: torch.randn(*s, generator=g)
