@@ -15,7 +15,7 @@ weights with a cache and state of its own.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, replace
 from typing import Any, Mapping, Optional
 
 from .errors import UnsupportedModelError
@@ -107,15 +107,23 @@ class ZarinexConfig:
         if not isinstance(layers, list) or not layers:
             raise UnsupportedModelError("layers must be a list with at least one layer")
         norm = _need(raw, "norm", "")
-        parsed = tuple(ZarinexLayer.parse(l, i) for i, l in enumerate(layers))
+        parsed = [ZarinexLayer.parse(l, i) for i, l in enumerate(layers)]
         for i, layer in enumerate(parsed):
             j = layer.weights_of
             if j is None:
                 continue
-            if not 0 <= j < len(parsed) or j == i or parsed[j].weights_of is not None:
-                raise UnsupportedModelError(f"layers[{i}].weights_of={j} must name another layer that has tensors of its own")
+            # a layer that names one which itself runs another's tensors runs those: follow to the owner
+            seen = {i}
+            while isinstance(j, int) and 0 <= j < len(parsed) and j not in seen and parsed[j].weights_of is not None:
+                seen.add(j)
+                j = parsed[j].weights_of
+            if not 0 <= j < len(parsed) or j in seen:
+                raise UnsupportedModelError(f"layers[{i}].weights_of={layer.weights_of} must lead to another layer that has tensors of its own")
             if (parsed[j].type, dict(parsed[j].mixer), parsed[j].mlp) != (layer.type, dict(layer.mixer), layer.mlp):
                 raise UnsupportedModelError(f"layers[{i}] runs the weights of layers[{j}] but differs from it in its sizes")
+            if j != layer.weights_of:
+                parsed[i] = replace(layer, weights_of=j)
+        parsed = tuple(parsed)
         return cls(vocab=_positive(_need(raw, "vocab", ""), "vocab"), width=_positive(_need(raw, "width", ""), "width"),
                    norm_eps=float(_need(norm, "eps", "norm")), postln_alpha=float(raw.get("postln_alpha", 1.0)),
                    layers=parsed)

@@ -39,6 +39,14 @@ def build(raw):
     return cfg, Model(arch.build_spec(cfg), Runtime(torch.device("cpu"), torch.float32))
 
 
+def test_a_layer_that_names_a_borrower_runs_the_owners_tensors():
+    raw = cfg_dict()
+    raw["layers"].append({"type": "mamba1", "mixer": raw["layers"][0]["mixer"], "mlp": raw["layers"][0]["mlp"], "weights_of": 4})
+    cfg, model = build(raw)
+    assert [l.weights_of for l in cfg.layers] == [None, None, None, 1, 0, 0]
+    assert [e.layer for e in model.spec.schedule] == [0, 1, 2, 1, 0, 0]
+
+
 def test_config_is_read_and_becomes_parts():
     from dli_amd.parts import CompositeCacheSpec, PagedKVSpec, StateSpec
 
@@ -105,7 +113,8 @@ def test_what_is_not_implemented_is_refused():
     broken(lambda r: r["layers"][0]["mlp"].__setitem__("kind", "dense"))
     broken(lambda r: r["layers"][0]["mlp"]["router"].__setitem__("top", 8))          # more than there are experts
     broken(lambda r: r["layers"][3].__setitem__("weights_of", 3))                     # itself
-    broken(lambda r: r["layers"][3].__setitem__("weights_of", 4))                     # a layer without tensors
+    broken(lambda r: r["layers"][3].__setitem__("weights_of", 4))                     # leads to a layer of another kind
+    broken(lambda r: (r["layers"][0].__setitem__("weights_of", 4), None))             # 0 -> 4 -> 0: nobody has the tensors
     broken(lambda r: r["layers"][3].__setitem__("weights_of", 2))                     # a layer of another kind
     broken(lambda r: r["layers"][3].__setitem__("weights_of", "1"))
     broken(lambda r: r["layers"][4].__setitem__("mixer", dict(r["layers"][4]["mixer"], inner=44)))               # other sizes than its source
