@@ -1,3 +1,3 @@
 """Architectures that ship with the engine. Importing this package registers them."""
 
-from . import llama, makodra, miberax, zarinex  # noqa: F401
+from . import betepel, llama, makodra, miberax, zarinex  # noqa: F401

@@ -83,7 +83,7 @@ def bytes_per_page(groups: Sequence[PagedKVSpec], layers_per_group: Sequence[int
                    dtype: torch.dtype) -> int:
     """Bytes that one page id costs across all groups and layers, keys and values."""
     item = torch.empty((), dtype=dtype).element_size()
-    return sum(n * page_size * g.kv_heads * (g.head_dim + g.v_dim) * item for g, n in zip(groups, layers_per_group))
+    return sum(n * page_size * (g.kv_heads * g.head_dim + g.v_heads * g.v_dim) * item for g, n in zip(groups, layers_per_group))
 
 
 class CacheStore:
@@ -98,7 +98,7 @@ class CacheStore:
         # per group: the tensors [layers, 1 or 2, pages, elements] that hold its pages
         self.pools: list[list[torch.Tensor]] = []
         for g, n_layers in zip(self.groups, self.layers_per_group):
-            sizes = [g.kv_heads * page_size * g.head_dim, g.kv_heads * page_size * g.v_dim]
+            sizes = [g.kv_heads * page_size * g.head_dim, g.v_heads * page_size * g.v_dim]
             if sizes[0] == sizes[1]:
                 shapes = [(n_layers, 2, num_pages, sizes[0])]
             else:
@@ -121,7 +121,7 @@ class CacheStore:
                 return LayerCache(
                     "paged", g,
                     keys.view(num_pages, spec.kv_heads, page_size, spec.head_dim),
-                    None if values is None else values.view(num_pages, spec.kv_heads, spec.v_dim, page_size),
+                    None if values is None else values.view(num_pages, spec.v_heads, spec.v_dim, page_size),
                     window=spec.window)
             if isinstance(spec, StateSpec):
                 return LayerCache(

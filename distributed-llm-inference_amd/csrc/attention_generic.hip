@@ -20,7 +20,11 @@
 //                 value, so a row's weights may add up to less than one;
 //   value_dim     the size of a value where it differs from a key's;
 //   gate          float32 [tokens][gate_stride]: the result is multiplied by sigmoid(gate) element
-//                 by element (same layout as the output).
+//                 by element (same layout as the output);
+//   keep_first    with a window: keys at positions below keep_first stay visible however far back they lie;
+//   v_heads       the value pages hold v_heads heads, a divisor of kv_heads, and kv head g reads the values of
+//                 head g % v_heads (several score maps over one set of values);
+//   out32         float32 [tokens][out_stride]: the result goes there unrounded instead of to `out`.
 // tile_entry == nullptr: every entry is a single row (steps of single tokens, whose launches read
 // nothing that the host made from the step's lengths); a kernel of its own takes these, below.
 //
@@ -35,6 +39,9 @@ struct ScoreChanges {
   int value_dim;
   const float* gate;
   int64_t gate_stride;
+  int keep_first;
+  int v_heads;
+  float* out32;
 };
 
 template <typename T, int RM, int RN, int DC>
@@ -58,6 +65,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   const int value_dim = sc.value_dim;
   const float r1 = sc.r1 != nullptr ? sc.r1[head] : 0.f, r2 = sc.r1 != nullptr ? sc.r2[head] : 0.f;
   const int kvh = head / (q_heads / kv_heads);
+  const int vh = kvh % sc.v_heads;
   const int tok0 = q_start[entry];
   const int q_len = q_start[entry + 1] - tok0;
   const int n_keys = kv_len[entry];
@@ -80,13 +88,16 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
   }
 
   const int pos_lo = first_pos + q0, pos_hi = first_pos + q0 + rows - 1;
-  int j_begin = 0;
-  if (window > 0) j_begin = max(0, pos_lo - window + 1);
-  if (sc.chunk > 0) j_begin = max(j_begin, pos_lo / sc.chunk * sc.chunk);
+  int j_lo = sc.chunk > 0 ? pos_lo / sc.chunk * sc.chunk : 0;   // nothing before it is seen
+  int j_begin = j_lo;
+  if (window > 0) j_begin = max(j_lo, pos_lo - window + 1);
   j_begin = j_begin / BN * BN;
+  j_lo = j_lo / BN * BN;
+  const int keep = window > 0 ? sc.keep_first : 0;              // keys below it are seen from any distance
   const int j_end = rows > 0 ? pos_hi + 1 : 0;
 
-  for (int j0 = j_begin; j0 < j_end; j0 += BN) {
+  for (int j0 = keep > j_lo ? j_lo : j_begin; j0 < j_end; j0 += BN) {
+    if (j0 >= keep && j0 < j_begin) j0 = j_begin;               // between the kept keys and the window: nothing
     __syncthreads();  // previous tile's reads of ks/vs/ps are done (and qs is written)
     for (int idx = tid; idx < BN * head_dim; idx += 256) {
       const int r = idx / head_dim, c = idx - r * head_dim;
@@ -104,7 +115,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       float vv = 0.f;
       if (j < j_end) {
         const int64_t page = table[j / page_size];
-        vv = to_f32(v_pages[((page * kv_heads + kvh) * value_dim + c) * page_size + j % page_size]);
+        vv = to_f32(v_pages[((page * sc.v_heads + vh) * value_dim + c) * page_size + j % page_size]);
       }
       vs[r][c] = vv;
     }
@@ -135,7 +146,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
 #pragma unroll
       for (int jj = 0; jj < RN; ++jj) {
         const int j = j0 + tx + 16 * jj;
-        const bool visible = r < rows && j <= pos && (window <= 0 || j > pos - window) &&
+        const bool visible = r < rows && j <= pos && (window <= 0 || j > pos - window || j < sc.keep_first) &&
                              (sc.chunk <= 0 || j / sc.chunk == pos / sc.chunk);
         if (sc.r1 != nullptr && visible) s[i][jj] -= r1 * log1pf(r2 * (float)(pos - j));
         s[i][jj] = visible ? s[i][jj] : -INFINITY;
@@ -194,7 +205,8 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       if (tx + 16 * c < value_dim) {
         float y = acc[i][c] * inv;
         if (g != nullptr) y *= 1.f / (1.f + expf(-g[tx + 16 * c]));
-        o[tx + 16 * c] = from_f32<T>(y);
+        if (sc.out32 != nullptr) sc.out32[(int64_t)(tok0 + q0 + r) * out_stride + (int64_t)head * value_dim + tx + 16 * c] = y;
+        else o[tx + 16 * c] = from_f32<T>(y);
       }
   }
 }
@@ -241,6 +253,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
   float* ms = ps + waves * GQ * 64;              // [waves][GQ] reference points, then [waves][GQ] sums
   float* accs = ms + 2 * waves * GQ;             // [waves][GQ][VC * 64]
   const int entry = blockIdx.x / splits, split = blockIdx.x % splits, kvh = blockIdx.y;
+  const int vh = kvh % sc.v_heads;
   const int group = q_heads / kv_heads;
   const int h0 = kvh * group + blockIdx.z * GQ;                  // first query head of this workgroup
   const int nh = min(GQ, kvh * group + group - h0);              // heads that exist
@@ -262,16 +275,22 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
 #pragma unroll
     for (int c = 0; c < VC; ++c) acc[h][c] = 0.f;
   }
-  int j_begin = 0;
-  if (window > 0) j_begin = max(0, pos - window + 1);
-  if (sc.chunk > 0) j_begin = max(j_begin, pos / sc.chunk * sc.chunk);
+  const int j_lo = sc.chunk > 0 ? pos / sc.chunk * sc.chunk : 0;   // nothing before it is seen
+  int j_begin = j_lo;
+  if (window > 0) j_begin = max(j_lo, pos - window + 1);
+  const int keep = window > 0 ? sc.keep_first : 0;                 // keys below it are seen from any distance
+  // the blocks of 64 keys that hold something visible: those of the kept keys that lie before the window's, then the window's
+  const int b_win = j_begin / 64;
+  const int nb_keep = keep > j_lo ? max(min((keep + 63) / 64, b_win) - j_lo / 64, 0) : 0;
+  const int nb_all = nb_keep + pos / 64 - b_win + 1;
   __syncthreads();
 
   const bool k_packs = head_dim % PN == 0, v_packs = page_size % PN == 0;
   // blocks of 64 keys go round the waves of the `splits` workgroups that share this (entry, heads)
-  for (int j0 = j_begin / 64 * 64 + (split * waves + wave) * 64; j0 <= pos; j0 += 64 * waves * splits) {
+  for (int b = split * waves + wave; b < nb_all; b += waves * splits) {
+    const int j0 = (b < nb_keep ? j_lo / 64 + b : b_win + b - nb_keep) * 64;
     const int j = j0 + lane;
-    const bool seen = j >= j_begin && j <= pos;
+    const bool seen = j <= pos && j >= j_lo && (j >= j_begin || j < keep);
     // the page of this lane's key, for its own row of K and, handed round, for the rows of V (a key
     // past the request's last page reads the table's last entry: its weight is zero)
     const int my_page = table[min(j / page_size, table_stride - 1)];
@@ -319,7 +338,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     // lanes are value columns now
     const int last = min(63, pos - j0);
-    const int first = max(0, j_begin - j0);
+    const int first = keep > 0 ? 0 : max(0, j_begin - j0);   // (keys that are not seen weigh nothing)
     if (v_packs) {
       // every pack of the block's 64 keys is asked for before the first is used; keys that are not
       // seen have weight zero and lie in pages that exist (or in the table's last entry's page)
@@ -331,7 +350,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
 #pragma unroll
         for (int k = 0; k < PACKS; ++k) {
           const int64_t page = __shfl(my_page, k * PN, DLI_WAVE);
-          vv[k] = *reinterpret_cast<const P16*>(v_pages + ((page * kv_heads + kvh) * value_dim + col) * page_size +
+          vv[k] = *reinterpret_cast<const P16*>(v_pages + ((page * sc.v_heads + vh) * value_dim + col) * page_size +
                                                 (j0 + k * PN) % page_size);
         }
 #pragma unroll
@@ -355,7 +374,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
           const int jk = j0 + jj;
           const int64_t page = table[jk / page_size];
           const int off = jk % page_size;
-          const T* vr = v_pages + ((page * kv_heads + kvh) * value_dim + col) * page_size + off;
+          const T* vr = v_pages + ((page * sc.v_heads + vh) * value_dim + col) * page_size + off;
           if (v_packs && off % PN == 0 && jj + PN - 1 <= last) {
             const P16 vv = *reinterpret_cast<const P16*>(vr);
 #pragma unroll
@@ -415,7 +434,8 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
     float y = l > 0.f ? o / l : 0.f;
     const int64_t at = (int64_t)(h0 + h) * value_dim + col;
     if (sc.gate != nullptr) y *= 1.f / (1.f + expf(-sc.gate[(int64_t)entry * sc.gate_stride + at]));
-    out[(int64_t)entry * out_stride + at] = from_f32<T>(y);
+    if (sc.out32 != nullptr) sc.out32[(int64_t)entry * out_stride + at] = y;
+    else out[(int64_t)entry * out_stride + at] = from_f32<T>(y);
   }
 }
 
@@ -424,7 +444,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
 template <typename T>
 __global__ void attention_scored_merge_kernel(const float* __restrict__ parts, int splits, int q_heads, int value_dim,
                                               const float* __restrict__ gate, int64_t gate_stride, T* __restrict__ out,
-                                              int64_t out_stride) {
+                                              int64_t out_stride, float* __restrict__ out32) {
   const int entry = blockIdx.x, head = blockIdx.y;
   const float* base = parts + ((int64_t)entry * q_heads + head) * splits * (value_dim + 2);
   float m = -INFINITY;
@@ -442,7 +462,8 @@ __global__ void attention_scored_merge_kernel(const float* __restrict__ parts, i
     float y = l > 0.f ? o / l : 0.f;
     const int64_t at = (int64_t)head * value_dim + col;
     if (gate != nullptr) y *= 1.f / (1.f + expf(-gate[(int64_t)entry * gate_stride + at]));
-    out[(int64_t)entry * out_stride + at] = from_f32<T>(y);
+    if (out32 != nullptr) out32[(int64_t)entry * out_stride + at] = y;
+    else out[(int64_t)entry * out_stride + at] = from_f32<T>(y);
   }
 }
 
@@ -476,7 +497,7 @@ static int launch_scored_decode(const void* q, int64_t q_stride, const void* k_p
     if (status != DLI_OK) return status;
     attention_scored_merge_kernel<T><<<dim3(entries, q_heads), sc.value_dim <= 64 ? 64 : sc.value_dim <= 128 ? 128 : 256, 0,
                                        stream>>>(parts, splits, q_heads, sc.value_dim, sc.gate, sc.gate_stride, (T*)out,
-                                                 out_stride);
+                                                 out_stride, sc.out32);
   }
   return dli_launch_status();
 }
@@ -497,15 +518,18 @@ static int attention_scored(const void* q, int64_t q_stride, const void* k_pages
                             int tiles, int q_heads, int kv_heads, int head_dim, int value_dim,
                             int page_size, float scale, int window, int chunk, int sink,
                             const float* r1, const float* r2, const float* gate,
-                            int64_t gate_stride, float* parts, int splits, int is_bf16, hipStream_t stream) {
+                            int64_t gate_stride, int keep_first, int v_heads, float* out32, float* parts, int splits,
+                            int is_bf16, hipStream_t stream) {
   if (tiles <= 0) return DLI_OK;
+  if (v_heads <= 0) v_heads = kv_heads;
+  if (keep_first < 0 || kv_heads <= 0 || kv_heads % v_heads != 0) return DLI_ERR_ARGUMENT;
   const int dmax = head_dim > value_dim ? head_dim : value_dim;
   if (head_dim <= 0 || value_dim <= 0 || dmax > 256 || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || q_heads > 65535 || page_size <= 0 || table_stride <= 0 ||
       window < 0 || chunk < 0 || (r1 == nullptr) != (r2 == nullptr) ||
       (tile_entry == nullptr) != (tile_q0 == nullptr))
     return DLI_ERR_ARGUMENT;
-  const ScoreChanges sc = {chunk, sink, r1, r2, value_dim, gate, gate_stride};
+  const ScoreChanges sc = {chunk, sink, r1, r2, value_dim, gate, gate_stride, keep_first, v_heads, out32};
   if (tile_entry == nullptr) {
     // every entry is one row: the kernel whose lanes own keys, then value columns
     const int group = q_heads / kv_heads;
@@ -543,10 +567,11 @@ extern "C" int dli_attention_scored(const void* q, int64_t q_stride, const void*
                                     int tiles, int q_heads, int kv_heads, int head_dim, int value_dim,
                                     int page_size, float scale, int window, int chunk, int sink,
                                     const float* r1, const float* r2, const float* gate,
-                                    int64_t gate_stride, int is_bf16, hipStream_t stream) {
+                                    int64_t gate_stride, int keep_first, int v_heads, float* out32, int is_bf16,
+                                    hipStream_t stream) {
   return attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len, block_tables, table_stride,
                           tile_entry, tile_q0, tiles, q_heads, kv_heads, head_dim, value_dim, page_size, scale, window,
-                          chunk, sink, r1, r2, gate, gate_stride, nullptr, 1, is_bf16, stream);
+                          chunk, sink, r1, r2, gate, gate_stride, keep_first, v_heads, out32, nullptr, 1, is_bf16, stream);
 }
 
 // How many workgroups share the keys of an (entry, group of query heads) in a step of single tokens: as
@@ -568,11 +593,12 @@ extern "C" int dli_attention_scored_single(const void* q, int64_t q_stride, cons
                                            int table_stride, int entries, int q_heads, int kv_heads, int head_dim,
                                            int value_dim, int page_size, float scale, int window, int chunk, int sink,
                                            const float* r1, const float* r2, const float* gate, int64_t gate_stride,
-                                           float* parts, int splits, int is_bf16, hipStream_t stream) {
+                                           int keep_first, int v_heads, float* out32, float* parts, int splits,
+                                           int is_bf16, hipStream_t stream) {
   if (splits < 1 || splits > 64 || (splits > 1 && parts == nullptr)) return DLI_ERR_ARGUMENT;
   return attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, nullptr, kv_len, block_tables, table_stride,
                           nullptr, nullptr, entries, q_heads, kv_heads, head_dim, value_dim, page_size, scale, window,
-                          chunk, sink, r1, r2, gate, gate_stride, parts, splits, is_bf16, stream);
+                          chunk, sink, r1, r2, gate, gate_stride, keep_first, v_heads, out32, parts, splits, is_bf16, stream);
 }
 
 extern "C" int dli_attention_generic(const void* q, int64_t q_stride, const void* k_pages,
@@ -585,5 +611,5 @@ extern "C" int dli_attention_generic(const void* q, int64_t q_stride, const void
   return attention_scored(q, q_stride, k_pages, v_pages, out, out_stride, q_start, kv_len,
                           block_tables, table_stride, tile_entry, tile_q0, tiles, q_heads,
                           kv_heads, head_dim, head_dim, page_size, scale, window, 0, 0, nullptr,
-                          nullptr, nullptr, 0, nullptr, 1, is_bf16, stream);
+                          nullptr, nullptr, 0, 0, kv_heads, nullptr, nullptr, 1, is_bf16, stream);
 }

@@ -1,7 +1,8 @@
 // Attention with changed scores for the portions of a bfloat16 step, on the matrix cores.
 //
 // The same scores as csrc/attention_generic.hip (chunked mask, window, per-head logarithmic distance
-// penalty, sink, values of another size than keys, sigmoid gate), computed with
+// penalty, sink, values of another size than keys, sigmoid gate, kept first keys, value heads shared by
+// several key heads, an unrounded result), computed with
 // v_mfma_f32_16x16x16_bf16 in transposed form, S^T = K Q^T and O^T = V^T P^T: a lane then holds four
 // consecutive keys' scores of ONE query (query = lane % 16), so the running maximum, the sum and the
 // rescaling of a query stay in its four lanes, and the result of the first product is, lane by lane,
@@ -31,6 +32,8 @@ struct ScoredArgs {
   float scale; int window, chunk, sink;
   const float* r1; const float* r2;
   const float* gate; int64_t gate_stride;
+  int keep_first, v_heads;
+  float* out32;
 };
 
 template <int DT, int VT>   // head_dim = 16 DT, value_dim = 16 VT
@@ -48,7 +51,7 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
   const bool q_live = qrow0 + col < q_len;
   const int my_q = min(qrow0 + col, q_len - 1);
   const int pos = first_pos + my_q;
-  const int ps = a.page_size, G = a.kv_heads;
+  const int ps = a.page_size, G = a.kv_heads, GV = a.v_heads, vh = kvh % a.v_heads;
   const int* table = a.block_tables + (int64_t)entry * a.table_stride;
 
   short4s qb[DT];   // Q^T: dims 16 d + 4 grp .. + 3 of this lane's query
@@ -60,10 +63,12 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
   const float r1 = a.r1 != nullptr ? a.r1[head] : 0.f, r2 = a.r1 != nullptr ? a.r2[head] : 0.f;
   const float scale2 = a.scale * LOG2E;
   const int p_lo = first_pos + qrow0, p_hi = first_pos + min(qrow0 + 15, q_len - 1);
-  int j_begin = 0;
-  if (a.window > 0) j_begin = max(0, p_lo - a.window + 1);
-  if (a.chunk > 0) j_begin = max(j_begin, p_lo / a.chunk * a.chunk);
+  int j_lo = a.chunk > 0 ? p_lo / a.chunk * a.chunk : 0;        // nothing before it is seen
+  int j_begin = j_lo;
+  if (a.window > 0) j_begin = max(j_lo, p_lo - a.window + 1);
   j_begin = j_begin / 64 * 64;
+  j_lo = j_lo / 64 * 64;
+  const int keep = a.window > 0 ? a.keep_first : 0;             // keys below it are seen from any distance
   const int my_chunk = a.chunk > 0 ? pos / a.chunk : 0;
 
   float4s acc[VT];
@@ -72,7 +77,8 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
   float m_run = a.sink ? 0.f : -INFINITY;              // the sink: a key of score 0 without a value,
   float l_run = a.sink && grp == 0 ? 1.f : 0.f;        // counted once a query (sums are per lane until the end)
 
-  for (int j0 = j_begin; j0 <= p_hi; j0 += 64) {
+  for (int j0 = keep > j_lo ? j_lo : j_begin; j0 <= p_hi; j0 += 64) {
+    if (j0 >= keep && j0 < j_begin) j0 = j_begin;               // between the kept keys and the window: nothing
     float4s s[4];
 #pragma unroll
     for (int sub = 0; sub < 4; ++sub) {
@@ -91,7 +97,7 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int j = j0 + 16 * sub + 4 * grp + i;
-        const bool seen = q_live && j <= pos && (a.window <= 0 || j > pos - a.window) &&
+        const bool seen = q_live && j <= pos && (a.window <= 0 || j > pos - a.window || j < a.keep_first) &&
                           (a.chunk <= 0 || j / a.chunk == my_chunk);
         float x = s[sub][i] * scale2;
         if (a.r1 != nullptr) x -= r1 * __builtin_amdgcn_logf(1.f + r2 * (float)max(pos - j, 0));
@@ -123,7 +129,7 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
     for (int sub = 0; sub < 4; ++sub) {
       const int key = j0 + 16 * sub + 4 * grp;          // the four keys whose values this lane reads, one value row a product
       const int64_t page = table[min(key / ps, a.table_stride - 1)];
-      const bf16_t* vr = a.v_pages + ((page * G + kvh) * V + col) * ps + key % ps;
+      const bf16_t* vr = a.v_pages + ((page * GV + vh) * V + col) * ps + key % ps;
 #pragma unroll
       for (int t = 0; t < VT; ++t)
         acc[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(*reinterpret_cast<const short4s*>(vr + (int64_t)16 * t * ps),
@@ -140,14 +146,17 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
   for (int t = 0; t < VT; ++t) {
     const int64_t at = (int64_t)head * V + 16 * t + 4 * grp;
     short4s o;
+    float4s of;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float y = acc[t][i] * inv;
       if (a.gate != nullptr) y *= 1.f / (1.f + __expf(-a.gate[row * a.gate_stride + at + i]));
+      of[i] = y;
       const bf16_t yb = (bf16_t)y;
       o[i] = *reinterpret_cast<const short*>(&yb);
     }
-    *reinterpret_cast<short4s*>(a.out + row * a.out_stride + at) = o;
+    if (a.out32 != nullptr) *reinterpret_cast<float4s*>(a.out32 + row * a.out_stride + at) = of;
+    else *reinterpret_cast<short4s*>(a.out + row * a.out_stride + at) = o;
   }
 }
 
@@ -183,8 +192,10 @@ extern "C" int dli_attention_scored_mfma(const void* q, int64_t q_stride, const 
                                          const int* tile_q0, int tiles, int q_heads, int kv_heads, int head_dim,
                                          int value_dim, int page_size, float scale, int window, int chunk, int sink,
                                          const float* r1, const float* r2, const float* gate, int64_t gate_stride,
-                                         hipStream_t stream) {
+                                         int keep_first, int v_heads, float* out32, hipStream_t stream) {
   if (tiles <= 0) return DLI_OK;
+  if (v_heads <= 0) v_heads = kv_heads;
+  if (keep_first < 0 || kv_heads <= 0 || kv_heads % v_heads != 0) return DLI_ERR_ARGUMENT;
   if (!dli_attention_scored_mfma_supports(head_dim, value_dim, page_size) || q_heads <= 0 || kv_heads <= 0 ||
       q_heads % kv_heads != 0 || q_heads > 65535 || table_stride <= 0 || window < 0 || chunk < 0 ||
       (r1 == nullptr) != (r2 == nullptr) || tile_entry == nullptr || tile_q0 == nullptr || q_stride % 4 != 0 ||
@@ -196,6 +207,7 @@ extern "C" int dli_attention_scored_mfma(const void* q, int64_t q_stride, const 
   a.block_tables = block_tables; a.table_stride = table_stride; a.tile_entry = tile_entry; a.tile_q0 = tile_q0;
   a.q_heads = q_heads; a.kv_heads = kv_heads; a.page_size = page_size; a.scale = scale; a.window = window;
   a.chunk = chunk; a.sink = sink; a.r1 = r1; a.r2 = r2; a.gate = gate; a.gate_stride = gate_stride;
+  a.keep_first = keep_first; a.v_heads = v_heads; a.out32 = out32;
   switch (head_dim / 16) {
     case 1: return launch_scored_mfma<1>(a, tiles, value_dim, stream);
     case 2: return launch_scored_mfma<2>(a, tiles, value_dim, stream);

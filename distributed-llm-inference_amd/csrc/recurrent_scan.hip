@@ -235,19 +235,22 @@ __global__ void recurrent_scan_any_kernel(ScanArgs p, int D) {
 }
 
 // out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre), head by head: a wave a (row, head).
+// den (may be nullptr) float32 [rows][heads]: o is divided by it first, head by head.
 template <typename T, int RULE>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, int64_t o_stride,
                                                              const float* __restrict__ g_pre, int64_t g_stride,
                                                              const float* __restrict__ norm_w, float eps,
-                                                             T* __restrict__ out, int64_t out_stride, int heads, int dim) {
+                                                             T* __restrict__ out, int64_t out_stride, int heads, int dim,
+                                                             const float* __restrict__ den) {
   const int64_t row = blockIdx.x;
   const int lane = threadIdx.x % DLI_WAVE, wave = threadIdx.x / DLI_WAVE;
   const int h = blockIdx.y * 4 + wave;
   if (h < heads) {
     const float* oh = o + row * o_stride + (int64_t)h * dim;
+    const float dn = den != nullptr ? 1.f / den[row * heads + h] : 1.f;
     float ss = 0.f;
-    for (int c = lane; c < dim; c += DLI_WAVE) ss += oh[c] * oh[c];
-    const float r = 1.f / sqrtf(wave_sum(ss) / (float)dim + eps);
+    for (int c = lane; c < dim; c += DLI_WAVE) ss += (oh[c] * dn) * (oh[c] * dn);
+    const float r = dn / sqrtf(wave_sum(ss) / (float)dim + eps);
     for (int c = lane; c < dim; c += DLI_WAVE) {
       float gate = 1.f;                                   // RULE 2: no gate (g_pre is not read)
       if (RULE != GATE_NONE) {
@@ -284,10 +287,10 @@ static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int ou
   if (dli_launch_status() != DLI_OK) return DLI_ERR_LAUNCH;
   if (out_is_bf16)
     head_norm_gate_kernel<bf16_t, RULE><<<dim3(rows, (p.heads + 3) / 4), 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
-                                                                  (bf16_t*)p.out, p.out_stride, p.heads, dim);
+                                                                  (bf16_t*)p.out, p.out_stride, p.heads, dim, nullptr);
   else
     head_norm_gate_kernel<float, RULE><<<dim3(rows, (p.heads + 3) / 4), 256, 0, stream>>>(p.o_raw, p.o_stride, p.g_pre, p.g_stride, p.norm_w, p.eps,
-                                                                 (float*)p.out, p.out_stride, p.heads, dim);
+                                                                 (float*)p.out, p.out_stride, p.heads, dim, nullptr);
   return dli_launch_status();
 }
 
@@ -326,7 +329,7 @@ extern "C" int dli_recurrent_scan(const float* r, int64_t r_stride, const float*
 // norm_w holds heads * dim values (a weight that the heads share is repeated by the caller).
 extern "C" int dli_head_norm_gate(const float* o, int64_t o_stride, const float* g_pre, int64_t g_stride,
                                   const float* norm_w, float eps, void* out, int64_t out_stride, int rows, int heads,
-                                  int dim, int gate, int out_is_bf16, hipStream_t stream) {
+                                  int dim, int gate, const float* den, int out_is_bf16, hipStream_t stream) {
   // gate: 0 sigmoid(g_pre), 1 silu(g_pre), 2 none
   if (rows <= 0) return DLI_OK;
   const int64_t width = (int64_t)heads * dim;
@@ -335,7 +338,7 @@ extern "C" int dli_head_norm_gate(const float* o, int64_t o_stride, const float*
     return DLI_ERR_ARGUMENT;
   const dim3 grid(rows, (heads + 3) / 4);
   if (grid.y > 65535) return DLI_ERR_ARGUMENT;
-#define HNG(T, RULE) head_norm_gate_kernel<T, RULE><<<grid, 256, 0, stream>>>(o, o_stride, g_pre, g_stride, norm_w, eps, (T*)out, out_stride, heads, dim)
+#define HNG(T, RULE) head_norm_gate_kernel<T, RULE><<<grid, 256, 0, stream>>>(o, o_stride, g_pre, g_stride, norm_w, eps, (T*)out, out_stride, heads, dim, den)
   if (out_is_bf16) { if (gate == GATE_NONE) HNG(bf16_t, GATE_NONE); else if (gate) HNG(bf16_t, RULE_BONUS); else HNG(bf16_t, RULE_DELTA); }
   else { if (gate == GATE_NONE) HNG(float, GATE_NONE); else if (gate) HNG(float, RULE_BONUS); else HNG(float, RULE_DELTA); }
 #undef HNG

@@ -464,6 +464,18 @@ __global__ void expert_combine_kernel(const int* __restrict__ ids, const float* 
   out[row * width + c] = sum;
 }
 
+// A router that is a table: the experts of a token are the row of `table` [vocabulary][top] at its token id,
+// each with the weight 1 / top. A thread a (token, choice).
+__global__ void table_choose_kernel(const int* __restrict__ table, const int* __restrict__ token_ids, int n, int top,
+                                    int vocab, int* __restrict__ ids, float* __restrict__ weights) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n * top) return;
+  const int t = i / top, j = i - t * top;
+  const int tok = min(max(token_ids[t], 0), vocab - 1);
+  ids[i] = table[(int64_t)tok * top + j];
+  weights[i] = 1.f / (float)top;
+}
+
 extern "C" {
 
 int dli_poly_norm(const float* z, int64_t z_stride, const float* coef, void* out, int64_t out_stride, int rows, int ff,
@@ -551,6 +563,14 @@ int dli_expert_combine(const int* ids, const float* weights, const float* z, con
   else
     expert_combine_kernel<float><<<grid, 256, 0, stream>>>(ids, weights, z, (const float*)h, h_stride, shared_gate, gate_stride,
                                                            shared, shared_stride, out, top, experts, width);
+  return dli_launch_status();
+}
+
+int dli_table_choose(const int* table, const int* token_ids, int n, int top, int vocab, int* ids, float* weights,
+                     hipStream_t stream) {
+  if (n <= 0) return DLI_OK;
+  if (top <= 0 || vocab <= 0 || (int64_t)n * top > 0x7fffffff) return DLI_ERR_ARGUMENT;
+  table_choose_kernel<<<(n * top + 255) / 256, 256, 0, stream>>>(table, token_ids, n, top, vocab, ids, weights);
   return dli_launch_status();
 }
 

@@ -22,6 +22,10 @@
 //                      its own root mean square; with delta: x += delta first, in place
 //   branch_norm_mean   the mean of up to four branches' outputs, each first divided by its root mean
 //                      square over the row and multiplied by its own weight
+//   branch_weighted_sum  the sum of up to four branches' outputs, each times a constant of its own
+//   diff_head_norm     two attention maps over the same values combined head by head: a1 - lambda a2, divided by
+//                      its root mean square over the head, times a constant and a sigmoid gate per head
+//   scale_f32          y *= c in place
 #include "common.h"
 
 template <typename T>
@@ -250,25 +254,30 @@ __device__ __forceinline__ void rotary_cos_sin(float position, float freq, float
 // the given column offsets. The first rot_dims components of every q and k head are rotated by
 // position * inv_freq[i]: pair i is (2i, 2i+1) where `interleaved`, else (i, i + rot_dims/2); the
 // other components pass. q goes out in T; the rotated k and v go to the token's cache slot
-// (negative: not cached). A thread an element: it reads its partner from proj.
+// (negative: not cached). A thread an element: it reads its partner from proj. `bias` (may be nullptr)
+// holds a value for every column of proj and is added before anything else. The pages may hold fewer
+// value heads than key heads (v_heads), and none at all where the mixer reads another's (kv_heads 0).
 template <typename T>
 __global__ void rotary_cache_kernel(const float* __restrict__ proj, int64_t stride, int q_off, int k_off, int v_off,
+                                    const float* __restrict__ bias,
                                     const int* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dims,
                                     int interleaved, T* __restrict__ q_out, const int* __restrict__ slots,
-                                    T* __restrict__ k_pages, T* __restrict__ v_pages, int q_heads, int kv_heads, int dim,
-                                    int vdim, int page_size) {
+                                    T* __restrict__ k_pages, T* __restrict__ v_pages, int q_heads, int kv_heads, int v_heads,
+                                    int dim, int vdim, int page_size) {
   const int64_t row = blockIdx.x;
   const float* pr = proj + row * stride;
   const float p = (float)positions[row];
-  const int slot = slots[row];
+  const int slot = slots != nullptr ? slots[row] : -1;
   const int64_t page = slot >= 0 ? slot / page_size : 0;
   const int off = slot >= 0 ? slot % page_size : 0;
   const int half = rot_dims / 2;
   for (int i = threadIdx.x; i < (q_heads + kv_heads) * dim; i += blockDim.x) {
     const int h = i / dim, c = i - h * dim;
     const bool is_q = h < q_heads;
-    const float* src = is_q ? pr + q_off + (int64_t)h * dim : pr + k_off + (int64_t)(h - q_heads) * dim;
-    float y = src[c];
+    const int64_t at = is_q ? q_off + (int64_t)h * dim : k_off + (int64_t)(h - q_heads) * dim;
+    const float* src = pr + at;
+    const float* bs = bias != nullptr ? bias + at : nullptr;
+    float y = src[c] + (bs != nullptr ? bs[c] : 0.f);
     if (c < rot_dims) {
       int pair, partner;
       bool first;
@@ -276,16 +285,17 @@ __global__ void rotary_cache_kernel(const float* __restrict__ proj, int64_t stri
       else { first = c < half; pair = first ? c : c - half; partner = first ? c + half : c - half; }
       float cs, sn;
       rotary_cos_sin(p, inv_freq[pair], &cs, &sn);
-      const float other = src[partner];
+      const float other = src[partner] + (bs != nullptr ? bs[partner] : 0.f);
       y = first ? y * cs - other * sn : y * cs + other * sn;
     }
     if (is_q) q_out[(row * q_heads + h) * dim + c] = from_f32<T>(y);
     else if (slot >= 0) k_pages[((page * kv_heads + (h - q_heads)) * page_size + off) * dim + c] = from_f32<T>(y);
   }
   if (slot >= 0)
-    for (int i = threadIdx.x; i < kv_heads * vdim; i += blockDim.x) {
+    for (int i = threadIdx.x; i < v_heads * vdim; i += blockDim.x) {
       const int g = i / vdim, c = i - g * vdim;
-      v_pages[((page * kv_heads + g) * vdim + c) * page_size + off] = from_f32<T>(pr[v_off + i]);
+      v_pages[((page * v_heads + g) * vdim + c) * page_size + off] =
+          from_f32<T>(pr[v_off + i] + (bias != nullptr ? bias[v_off + i] : 0.f));
     }
 }
 
@@ -354,6 +364,47 @@ __global__ void branch_norm_mean_kernel(BranchArgs b, float* __restrict__ out, i
     for (int j = 0; j < COUNT; ++j) sum += b.weight[j][i] * (b.y[j][row * b.stride[j] + i] * r[j]);
     out[row * width + i] = sum * share;
   }
+}
+
+// Two attention maps over the same values become one result, head by head: with a1 = a[row][h] and
+// a2 = a[row][heads + h] (value_dim values each), d = a1 - lambda a2 is divided by its root mean square over the
+// head (no weight), multiplied by `after` and by sigmoid(gate[row][h]) (one number a head; nullptr: no gate).
+// A wave a (row, head).
+template <typename T>
+__global__ __launch_bounds__(256) void diff_head_norm_kernel(const float* __restrict__ a, int64_t a_stride, float lambda,
+                                                             float after, float eps, const float* __restrict__ gate,
+                                                             int64_t gate_stride, T* __restrict__ out, int64_t out_stride,
+                                                             int heads, int vdim) {
+  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x % DLI_WAVE, h = blockIdx.y * 4 + threadIdx.x / DLI_WAVE;
+  if (h >= heads) return;
+  const float* a1 = a + row * a_stride + (int64_t)h * vdim;
+  const float* a2 = a + row * a_stride + (int64_t)(heads + h) * vdim;
+  float ss = 0.f;
+  for (int c = lane; c < vdim; c += DLI_WAVE) {
+    const float d = a1[c] - lambda * a2[c];
+    ss += d * d;
+  }
+  float r = after / sqrtf(wave_sum(ss) / (float)vdim + eps);
+  if (gate != nullptr) r *= 1.f / (1.f + expf(-gate[row * gate_stride + h]));
+  for (int c = lane; c < vdim; c += DLI_WAVE)
+    out[row * out_stride + (int64_t)h * vdim + c] = from_f32<T>((a1[c] - lambda * a2[c]) * r);
+}
+
+// out = sum_b scale_b y_b for up to four float32 matrices of equal shape. A thread an element.
+struct WeightedBranches { const float* y[4]; int64_t stride[4]; float scale[4]; int count; };
+__global__ void branch_weighted_sum_kernel(WeightedBranches b, float* __restrict__ out, int width) {
+  const int64_t row = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  float sum = 0.f;
+  for (int j = 0; j < b.count; ++j) sum = fmaf(b.scale[j], b.y[j][row * b.stride[j] + i], sum);
+  out[row * width + i] = sum;
+}
+
+__global__ void scale_f32_kernel(float* __restrict__ y, int64_t n, float scale) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) y[i] *= scale;
 }
 
 extern "C" {
@@ -477,22 +528,23 @@ int dli_qk_unit_cache(const float* proj, int64_t stride, int q_off, int k_off, i
   return dli_launch_status();
 }
 
-int dli_rotary_cache(const float* proj, int64_t stride, int q_off, int k_off, int v_off, const int* positions,
-                     const float* inv_freq, int rot_dims, int interleaved, void* q_out, const int* slots, void* k_pages,
-                     void* v_pages, int rows, int q_heads, int kv_heads, int dim, int vdim, int page_size, int is_bf16,
-                     hipStream_t stream) {
+int dli_rotary_cache(const float* proj, int64_t stride, int q_off, int k_off, int v_off, const float* bias,
+                     const int* positions, const float* inv_freq, int rot_dims, int interleaved, void* q_out,
+                     const int* slots, void* k_pages, void* v_pages, int rows, int q_heads, int kv_heads, int v_heads,
+                     int dim, int vdim, int page_size, int is_bf16, hipStream_t stream) {
   if (rows <= 0) return DLI_OK;
-  if (q_heads <= 0 || kv_heads <= 0 || dim <= 0 || vdim <= 0 || page_size <= 0 || rot_dims < 0 || rot_dims > dim ||
-      rot_dims % 2 || (rot_dims > 0 && inv_freq == nullptr))
+  if (q_heads <= 0 || kv_heads < 0 || v_heads < 0 || dim <= 0 || vdim <= 0 || page_size <= 0 || rot_dims < 0 ||
+      rot_dims > dim || rot_dims % 2 || (rot_dims > 0 && inv_freq == nullptr) ||
+      (kv_heads > 0 && (k_pages == nullptr || slots == nullptr)) || (v_heads > 0 && (v_pages == nullptr || slots == nullptr)))
     return DLI_ERR_ARGUMENT;
   if (is_bf16)
-    rotary_cache_kernel<bf16_t><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, positions, inv_freq, rot_dims,
-                                                          interleaved, (bf16_t*)q_out, slots, (bf16_t*)k_pages,
-                                                          (bf16_t*)v_pages, q_heads, kv_heads, dim, vdim, page_size);
+    rotary_cache_kernel<bf16_t><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, bias, positions, inv_freq,
+                                                          rot_dims, interleaved, (bf16_t*)q_out, slots, (bf16_t*)k_pages,
+                                                          (bf16_t*)v_pages, q_heads, kv_heads, v_heads, dim, vdim, page_size);
   else
-    rotary_cache_kernel<float><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, positions, inv_freq, rot_dims,
-                                                         interleaved, (float*)q_out, slots, (float*)k_pages,
-                                                         (float*)v_pages, q_heads, kv_heads, dim, vdim, page_size);
+    rotary_cache_kernel<float><<<rows, 256, 0, stream>>>(proj, stride, q_off, k_off, v_off, bias, positions, inv_freq,
+                                                         rot_dims, interleaved, (float*)q_out, slots, (float*)k_pages,
+                                                         (float*)v_pages, q_heads, kv_heads, v_heads, dim, vdim, page_size);
   return dli_launch_status();
 }
 
@@ -527,6 +579,50 @@ int dli_branch_norm_mean(const float* const* y, const int64_t* strides, const fl
     case 3: branch_norm_mean_kernel<3><<<rows, 256, 0, stream>>>(b, out, width, eps); break;
     default: branch_norm_mean_kernel<4><<<rows, 256, 0, stream>>>(b, out, width, eps);
   }
+  return dli_launch_status();
+}
+
+int dli_diff_head_norm(const float* a, int64_t a_stride, float lambda, float after, float eps, const float* gate,
+                       int64_t gate_stride, void* out, int64_t out_stride, int rows, int heads, int vdim, int is_bf16,
+                       hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (heads <= 0 || vdim <= 0 || a_stride < (int64_t)2 * heads * vdim || out_stride < (int64_t)heads * vdim ||
+      (gate != nullptr && gate_stride < heads))
+    return DLI_ERR_ARGUMENT;
+  const dim3 grid(rows, (heads + 3) / 4);
+  if (grid.y > 65535) return DLI_ERR_ARGUMENT;
+  if (is_bf16)
+    diff_head_norm_kernel<bf16_t><<<grid, 256, 0, stream>>>(a, a_stride, lambda, after, eps, gate, gate_stride, (bf16_t*)out,
+                                                           out_stride, heads, vdim);
+  else
+    diff_head_norm_kernel<float><<<grid, 256, 0, stream>>>(a, a_stride, lambda, after, eps, gate, gate_stride, (float*)out,
+                                                          out_stride, heads, vdim);
+  return dli_launch_status();
+}
+
+int dli_branch_weighted_sum(const float* const* y, const int64_t* strides, const float* scales, int count, float* out,
+                            int rows, int width, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (count < 1 || count > 4 || width <= 0) return DLI_ERR_ARGUMENT;
+  WeightedBranches b;
+  b.count = count;
+  for (int j = 0; j < 4; ++j) {
+    b.y[j] = j < count ? y[j] : nullptr;
+    b.stride[j] = j < count ? strides[j] : 0;
+    b.scale[j] = j < count ? scales[j] : 0.f;
+    if (j < count && (y[j] == nullptr || strides[j] < width)) return DLI_ERR_ARGUMENT;
+  }
+  const dim3 grid(rows, (width + 255) / 256);
+  if (grid.y > 65535) return DLI_ERR_ARGUMENT;
+  branch_weighted_sum_kernel<<<grid, 256, 0, stream>>>(b, out, width);
+  return dli_launch_status();
+}
+
+int dli_scale_f32(float* y, int64_t n, float scale, hipStream_t stream) {
+  if (n <= 0) return DLI_OK;
+  const int64_t blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffff) return DLI_ERR_ARGUMENT;
+  scale_f32_kernel<<<(unsigned)blocks, 256, 0, stream>>>(y, n, scale);
   return dli_launch_status();
 }
 

@@ -99,15 +99,15 @@ _SIGNATURES = {
                               _c_int, _c_int, _c_ptr],
     "dli_attention_scored": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
-                             _c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
+                             _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_int, _c_ptr],
     "dli_attention_scored_splits": [_c_int, _c_int, _c_int],
     "dli_attention_scored_single": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                                     _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_i64,
-                                    _c_ptr, _c_int, _c_int, _c_ptr],
+                                    _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_attention_scored_mfma_supports": [_c_int, _c_int, _c_int],
     "dli_attention_scored_mfma": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_ptr,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_int, _c_ptr,
-                                  _c_ptr, _c_ptr, _c_i64, _c_ptr],
+                                  _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr],
     "dli_embed_sinusoid": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
     "dli_cast_from_f32": [_c_ptr, _c_ptr, _c_i64, _c_int, _c_ptr],
     "dli_norm_into_stream": [_c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
@@ -138,12 +138,22 @@ _SIGNATURES = {
     "dli_recurrent_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr,
                            _c_i64, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr,
                            _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
-    "dli_rotary_cache": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr,
-                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_rotary_cache": [_c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr,
+                         _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_diff_head_norm": [_c_ptr, _c_i64, _c_float, _c_float, _c_float, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_int, _c_int,
+                           _c_int, _c_int, _c_ptr],
+    "dli_branch_weighted_sum": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
+    "dli_scale_f32": [_c_ptr, _c_i64, _c_float, _c_ptr],
+    "dli_table_choose": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
+    "dli_exp_gates": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr,
+                      _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_scalar_gate_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
+                             _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int,
+                             _c_float, _c_int, _c_ptr],
     "dli_group_norm": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_branch_norm_mean": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_float, _c_ptr],
     "dli_head_norm_gate": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_float, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
-                           _c_int, _c_ptr],
+                           _c_ptr, _c_int, _c_ptr],
     "dli_gated_delta_max_taps": [],
     "dli_conv_prepare": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr,
                          _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr],
@@ -1566,22 +1576,28 @@ def attention_scored(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
                      q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
                      tile_entry: Optional[torch.Tensor], tile_q0: Optional[torch.Tensor], q_heads: int, scale: float,
                      *, window: int = 0, chunk: int = 0, sink: bool = False, r1: Optional[torch.Tensor] = None,
-                     r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+                     r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, keep_first: int = 0) -> None:
     """Paged causal attention on the vector units (32-bit arithmetic) with changes to the scores
-    as parameters: ``window`` and ``chunk`` restrict the keys a query sees, ``r1, r2`` (float32
+    as parameters: ``window`` and ``chunk`` restrict the keys a query sees (under a window the first
+    ``keep_first`` positions stay visible from any distance), ``r1, r2`` (float32
     ``[q_heads]``) take ``r1 log(1 + r2 (p - j))`` off the scaled score, ``sink`` adds ``exp(0)`` to the
     softmax's denominator, ``gate`` (float32 ``[tokens, q_heads*value_dim]``, rows contiguous)
-    multiplies the result by its sigmoid. Values may differ from keys in size (``v_pages``).
+    multiplies the result by its sigmoid. Values may differ from keys in size (``v_pages``), and the
+    value pages may hold fewer heads than the key pages, a divisor of their number: kv head ``g`` then
+    reads the values of head ``g % value_heads`` (several score maps over one set of values). ``out`` is
+    of the pages' type, or float32 (the result unrounded).
     Without tile lists every entry is one row (a step of single tokens)."""
     _dense(k_pages, "k_pages", ndim=4)
     dtype = k_pages.dtype
     _rows(q, "q", dtype)
-    _rows(out, "out", dtype)
+    out32 = out.dtype == torch.float32 and dtype != torch.float32
+    _rows(out, "out", torch.float32 if out32 else dtype)
     pages, kv_heads, page_size, head_dim = k_pages.shape
     _dense(v_pages, "v_pages", dtype, 4)
-    value_dim = v_pages.shape[2]
-    _require(v_pages.shape == (pages, kv_heads, value_dim, page_size),
-             "v_pages must be [pages, kv_heads, value_dim, page_size]")
+    v_heads, value_dim = v_pages.shape[1], v_pages.shape[2]
+    _require(v_pages.shape == (pages, v_heads, value_dim, page_size) and v_heads > 0 and kv_heads % v_heads == 0,
+             "v_pages must be [pages, value heads, value_dim, page_size], the value heads a divisor of the kv heads")
+    _require(keep_first >= 0, "keep_first must not be negative")
     _require(q.shape[1] == q_heads * head_dim and out.shape == (q.shape[0], q_heads * value_dim),
              "q must be [tokens, q_heads*head_dim] and out [tokens, q_heads*value_dim]")
     _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
@@ -1620,13 +1636,15 @@ def attention_scored(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tens
                 _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(kv_len),
                 _ptr(block_tables), block_tables.stride(0), entries, q_heads, kv_heads, head_dim, value_dim, page_size,
                 float(scale), int(window), int(chunk), int(bool(sink)), _ptr(r1), _ptr(r2), _ptr(gate), gate_stride,
-                _ptr(parts), splits, _is_bf16(dtype), _stream()), "attention_scored_single")
+                int(keep_first), v_heads, _ptr(out if out32 else None), _ptr(parts), splits, _is_bf16(dtype), _stream()),
+                "attention_scored_single")
             return
     _check(library().dli_attention_scored(
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
         _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tiles, q_heads, kv_heads,
         head_dim, value_dim, page_size, float(scale), int(window), int(chunk), int(bool(sink)), _ptr(r1), _ptr(r2),
-        _ptr(gate), gate_stride, _is_bf16(dtype), _stream()), "attention_scored")
+        _ptr(gate), gate_stride, int(keep_first), v_heads, _ptr(out if out32 else None), _is_bf16(dtype), _stream()),
+        "attention_scored")
 
 
 SCORED_MFMA_TILE_ROWS = 64  # queries of a tile of the matrix-core kernel (four waves of 16)
@@ -1641,25 +1659,27 @@ def attention_scored_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
                           q_start: torch.Tensor, kv_len: torch.Tensor, block_tables: torch.Tensor,
                           tile_entry: torch.Tensor, tile_q0: torch.Tensor, q_heads: int, scale: float, *,
                           window: int = 0, chunk: int = 0, sink: bool = False, r1: Optional[torch.Tensor] = None,
-                          r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None) -> None:
+                          r2: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, keep_first: int = 0) -> None:
     """:func:`attention_scored` for the portions of a bfloat16 step on the matrix cores: the same
     operands and parameters, tiles of ``SCORED_MFMA_TILE_ROWS`` queries, sizes that
     :func:`attention_scored_mfma_supports` takes."""
     _dense(k_pages, "k_pages", torch.bfloat16, 4)
     _rows(q, "q", torch.bfloat16)
-    _rows(out, "out", torch.bfloat16)
+    out32 = out.dtype == torch.float32
+    _rows(out, "out", torch.float32 if out32 else torch.bfloat16)
     pages, kv_heads, page_size, head_dim = k_pages.shape
     _dense(v_pages, "v_pages", torch.bfloat16, 4)
-    value_dim = v_pages.shape[2]
-    _require(v_pages.shape == (pages, kv_heads, value_dim, page_size),
-             "v_pages must be [pages, kv_heads, value_dim, page_size]")
+    v_heads, value_dim = v_pages.shape[1], v_pages.shape[2]
+    _require(v_pages.shape == (pages, v_heads, value_dim, page_size) and v_heads > 0 and kv_heads % v_heads == 0,
+             "v_pages must be [pages, value heads, value_dim, page_size], the value heads a divisor of the kv heads")
+    _require(keep_first >= 0, "keep_first must not be negative")
     _require(attention_scored_mfma_supports(head_dim, value_dim, page_size, k_pages.dtype),
              "the matrix-core kernel does not take these sizes")
     _require(q.shape[1] == q_heads * head_dim and out.shape == (q.shape[0], q_heads * value_dim),
              "q must be [tokens, q_heads*head_dim] and out [tokens, q_heads*value_dim]")
     _require(q_heads % kv_heads == 0, "query heads are not a multiple of kv heads")
-    _require(q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0 and q.data_ptr() % 8 == 0 and out.data_ptr() % 8 == 0,
-             "q and out must be 8-byte aligned, row by row")
+    _require(q.stride(0) % 4 == 0 and out.stride(0) % 4 == 0 and q.data_ptr() % 8 == 0
+             and out.data_ptr() % (16 if out32 else 8) == 0, "q and out must be aligned for four values at once, row by row")
     for name, t in (("q_start", q_start), ("kv_len", kv_len), ("tile_entry", tile_entry), ("tile_q0", tile_q0)):
         _dense(t, name, torch.int32, 1)
     _dense(block_tables, "block_tables", torch.int32, 2)
@@ -1681,7 +1701,8 @@ def attention_scored_mfma(q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch
         _ptr(q), q.stride(0), _ptr(k_pages), _ptr(v_pages), _ptr(out), out.stride(0), _ptr(q_start), _ptr(kv_len),
         _ptr(block_tables), block_tables.stride(0), _ptr(tile_entry), _ptr(tile_q0), tile_entry.shape[0], q_heads,
         kv_heads, head_dim, value_dim, page_size, float(scale), int(window), int(chunk), int(bool(sink)), _ptr(r1),
-        _ptr(r2), _ptr(gate), gate_stride, _stream()), "attention_scored_mfma")
+        _ptr(r2), _ptr(gate), gate_stride, int(keep_first), v_heads, _ptr(out if out32 else None), _stream()),
+        "attention_scored_mfma")
 
 
 RULE_DELTA, RULE_BONUS = 0, 1
@@ -1736,34 +1757,49 @@ def recurrent_scan(r: torch.Tensor, k: torch.Tensor, v: torch.Tensor, w: torch.T
 
 def rotary_cache(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, positions: torch.Tensor,
                  inv_freq: Optional[torch.Tensor], rot_dims: int, interleaved: bool, q_out: torch.Tensor,
-                 slots: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor, q_heads: int) -> None:
+                 slots: Optional[torch.Tensor], k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], q_heads: int,
+                 bias: Optional[torch.Tensor] = None) -> None:
     """From the float32 projections ``proj [n, >= ...]`` (q at ``q_off``, k at ``k_off``, v at ``v_off``):
     the first ``rot_dims`` components of every q and k head rotated by ``position * inv_freq[i]`` (pair
     ``i`` is ``(2i, 2i+1)`` where ``interleaved``, else ``(i, i + rot_dims/2)``; 32-bit angles),
-    ``q_out [n, q_heads*dim]``; rotated k and v written at each token's cache slot."""
+    ``q_out [n, q_heads*dim]``; rotated k and v written at each token's cache slot. ``bias`` (float32, a
+    value for every column of ``proj``) is added first. The value pages may hold fewer heads than the key
+    pages; without pages (``None``: the mixer reads another's) only q is made."""
     _f32_rows(proj, "proj")
-    _dense(k_pages, "k_pages", ndim=4)
-    dtype = k_pages.dtype
-    pages, kv_heads, page_size, dim = k_pages.shape
-    _dense(v_pages, "v_pages", dtype, 4)
-    vdim = v_pages.shape[2]
-    _require(v_pages.shape == (pages, kv_heads, vdim, page_size), "v_pages must be [pages, kv_heads, vdim, page_size]")
     n = proj.shape[0]
+    dtype = q_out.dtype
     _dense(q_out, "q_out", dtype, 2)
-    _require(q_out.shape == (n, q_heads * dim), "q_out must be [n, q_heads*dim]")
-    _dense(slots, "slots", torch.int32, 1)
+    _require(q_out.shape[0] == n and q_out.shape[1] % q_heads == 0, "q_out must be [n, q_heads*dim]")
+    dim = q_out.shape[1] // q_heads
+    kv_heads = v_heads = 0
+    page_size = vdim = 1
+    if k_pages is not None:
+        _dense(k_pages, "k_pages", dtype, 4)
+        pages, kv_heads, page_size, kdim = k_pages.shape
+        _require(kdim == dim, "keys and queries differ in size")
+        _dense(v_pages, "v_pages", dtype, 4)
+        v_heads, vdim = v_pages.shape[1], v_pages.shape[2]
+        _require(v_pages.shape == (pages, v_heads, vdim, page_size), "v_pages must be [pages, value heads, vdim, page_size]")
+        _dense(slots, "slots", torch.int32, 1)
+        _require(slots.shape[0] == n, "slots differ from proj in rows")
+    else:
+        _require(v_pages is None, "value pages come with key pages")
     _dense(positions, "positions", torch.int32, 1)
-    _require(slots.shape[0] == n and positions.shape[0] == n, "slots and positions differ from proj in rows")
-    for off, size in ((q_off, q_heads * dim), (k_off, kv_heads * dim), (v_off, kv_heads * vdim)):
+    _require(positions.shape[0] == n, "positions differ from proj in rows")
+    for off, size in ((q_off, q_heads * dim), (k_off, kv_heads * dim), (v_off, v_heads * vdim)):
         _require(0 <= off and off + size <= proj.shape[1], "a projection lies outside proj's columns")
+    if bias is not None:
+        _dense(bias, "bias", torch.float32, 1)
+        _require(bias.shape[0] >= max(q_off + q_heads * dim, k_off + kv_heads * dim, v_off + v_heads * vdim),
+                 "bias must hold a value for every projected column")
     _require(0 <= rot_dims <= dim and rot_dims % 2 == 0, "the rotated components must be an even number within the head")
     if rot_dims:
         _dense(inv_freq, "inv_freq", torch.float32, 1)
         _require(inv_freq.shape[0] * 2 == rot_dims, "inv_freq must hold rot_dims/2 frequencies")
     _check(library().dli_rotary_cache(
-        _ptr(proj), proj.stride(0), q_off, k_off, v_off, _ptr(positions), _ptr(inv_freq if rot_dims else None), int(rot_dims),
-        int(bool(interleaved)), _ptr(q_out), _ptr(slots), _ptr(k_pages), _ptr(v_pages), n, q_heads, kv_heads, dim, vdim,
-        page_size, _is_bf16(dtype), _stream()), "rotary_cache")
+        _ptr(proj), proj.stride(0), q_off, k_off, v_off, _ptr(bias), _ptr(positions), _ptr(inv_freq if rot_dims else None),
+        int(rot_dims), int(bool(interleaved)), _ptr(q_out), _ptr(slots if k_pages is not None else None), _ptr(k_pages),
+        _ptr(v_pages), n, q_heads, kv_heads, v_heads, dim, vdim, page_size, _is_bf16(dtype), _stream()), "rotary_cache")
 
 
 def group_norm(x: torch.Tensor, weight: torch.Tensor, groups: int, eps: float, out: torch.Tensor,
@@ -1871,7 +1907,7 @@ HEAD_GATES = {"sigmoid": 0, "silu": 1, "none": 2}
 
 
 def head_norm_gate(o: torch.Tensor, g_pre: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float, out: torch.Tensor,
-                   heads: int, dim: int, gate: str = "silu") -> None:
+                   heads: int, dim: int, gate: str = "silu", den: Optional[torch.Tensor] = None) -> None:
     """``out = o / sqrt(mean_head(o^2) + eps) * norm_w * gate(g_pre)`` head by head: ``o`` and ``g_pre`` float32
     ``[n, heads*dim]`` (rows contiguous), ``norm_w`` float32 ``[heads*dim]``, ``gate`` ``"silu"``, ``"sigmoid"`` or
     ``"none"`` (the per-head norm alone; ``g_pre`` is then ``None``)."""
@@ -1886,9 +1922,12 @@ def head_norm_gate(o: torch.Tensor, g_pre: Optional[torch.Tensor], norm_w: torch
         _require(g_pre.shape == (n, width), "g_pre must be [n, heads*dim]")
     _require(o.shape == (n, width) and out.shape == (n, width) and norm_w.shape[0] == width,
              "o, out and norm_w must be [n, heads*dim]")
+    if den is not None:   # every head of ``o`` is divided by its value first
+        _dense(den, "den", torch.float32, 2)
+        _require(den.shape == (n, heads), "den must be [n, heads]")
     _check(library().dli_head_norm_gate(_ptr(o), o.stride(0), _ptr(g_pre), 0 if g_pre is None else g_pre.stride(0),
                                         _ptr(norm_w), float(eps), _ptr(out), out.stride(0), n, heads, dim,
-                                        HEAD_GATES[gate], _is_bf16(out.dtype), _stream()), "head_norm_gate")
+                                        HEAD_GATES[gate], _ptr(den), _is_bf16(out.dtype), _stream()), "head_norm_gate")
 
 
 # ----------------------------------------------------------------------------- feed-forward: polynomial activation, experts
@@ -2182,3 +2221,116 @@ def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Opt
         g_stride = gate.stride(0)
     _check(library().dli_head_products(_ptr(x), x.stride(0), _ptr(w), _ptr(out), out.stride(0), _ptr(gate), g_stride, n,
                                        heads, m, k, _is_bf16(w.dtype), _stream()), "head_products")
+
+
+# ----------------------------------------------------------------------------- recurrences under scalar gates, differential maps
+
+def exp_gates(pre: torch.Tensor, i_off: int, f_off: int, i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor],
+              cap: float, state: torch.Tensor, m_off: int, q_start: torch.Tensor, positions: torch.Tensor,
+              state_slots: torch.Tensor, heads: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The factors of a matrix memory with exponential gates, per row and head of the step: from the float32
+    pre-activations ``pre [n, >=]`` (input gate of head ``h`` at column ``i_off + h``, forget gate at
+    ``f_off + h``; biases float32 ``[heads]``) the log gates ``i = cap tanh(. / cap)`` (``cap`` 0: as they are) and
+    ``f = logsigmoid(cap tanh(. / cap))``, the running reference point ``m <- max(f + m, i)`` (kept at
+    ``state[slot][m_off + h]``, 0 at position 0), and ``keep = exp(f + m_old - m)``, ``write = exp(i - m)``,
+    ``floor = exp(-m)``: three float32 ``[n, heads]``."""
+    _f32_rows(pre, "pre")
+    n = pre.shape[0]
+    _require(0 <= i_off and i_off + heads <= pre.shape[1] and 0 <= f_off and f_off + heads <= pre.shape[1],
+             "the gates lie outside pre's columns")
+    for name, t in (("i_bias", i_bias), ("f_bias", f_bias)):
+        if t is not None:
+            _dense(t, name, torch.float32, 1)
+            _require(t.shape[0] == heads, f"{name} must hold a value per head")
+    _state_rows(state, m_off + heads)
+    entries = _step_arrays(q_start, positions, state_slots, n)
+    out = torch.empty(3, n, heads, device=pre.device, dtype=torch.float32)
+    _check(library().dli_exp_gates(_ptr(pre), pre.stride(0), int(i_off), int(f_off), _ptr(i_bias), _ptr(f_bias), float(cap),
+                                   _ptr(state), state.stride(0), int(m_off), _ptr(q_start), _ptr(positions), _ptr(state_slots),
+                                   _ptr(out[0]), _ptr(out[1]), _ptr(out[2]), entries, n, heads, _stream()), "exp_gates")
+    return out[0], out[1], out[2]
+
+
+def scalar_gate_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor,
+                     positions: torch.Tensor, state_slots: torch.Tensor, o: torch.Tensor, heads: int, dim: int, vdim: int, *,
+                     keep: Optional[torch.Tensor] = None, write: Optional[torch.Tensor] = None,
+                     decay: Optional[torch.Tensor] = None, floor: Optional[torch.Tensor] = None,
+                     den: Optional[torch.Tensor] = None, q_scale: float = 1.0, silu: bool = False) -> None:
+    """Per request and head ``S <- a S + b k v^T``, ``o = S^T q`` over the step's rows in order, with
+    ``a, b = keep, write`` (float32 ``[n, heads]``) or ``a = decay[head]``, ``b = 1``. ``q, k [n, heads*dim]`` and
+    ``v [n, heads*vdim]`` are float32 with contiguous rows (columns of a wider matrix will do); with ``silu`` all
+    three pass through silu first; q is multiplied by ``q_scale``. With ``floor`` (float32 ``[n, heads]``) the state
+    has one more column a head, for a value that is always one, and ``den [n, heads]`` receives
+    ``max(|that column's result|, floor) + 1e-6``. ``S`` float32 ``[heads][vdim (+ 1)][dim]`` at the start of
+    ``state[slot]`` (zeros at position 0); ``o [n, heads*vdim]`` float32."""
+    for name, t, width in (("q", q, heads * dim), ("k", k, heads * dim), ("v", v, heads * vdim), ("o", o, heads * vdim)):
+        _f32_rows(t, name)
+        _require(t.shape[1] == width, f"{name} must hold {width} columns")
+    n = q.shape[0]
+    _require(k.shape[0] == n and v.shape[0] == n and o.shape[0] == n, "q, k, v and o differ in rows")
+    _require((keep is None) == (write is None) and (keep is not None or decay is not None), "keep and write, or decay")
+    _require((floor is None) == (den is None) and (floor is None or keep is not None), "floor and den come with the gates")
+    for name, t in (("keep", keep), ("write", write), ("floor", floor), ("den", den)):
+        if t is not None:
+            _dense(t, name, torch.float32, 2)
+            _require(t.shape == (n, heads), f"{name} must be [n, heads]")
+    if decay is not None:
+        _dense(decay, "decay", torch.float32, 1)
+        _require(decay.shape[0] == heads, "decay must hold a value per head")
+    _state_rows(state, heads * (vdim + (floor is not None)) * dim)
+    entries = _step_arrays(q_start, positions, state_slots, n)
+    _check(library().dli_scalar_gate_scan(
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(keep), _ptr(write), heads, _ptr(decay),
+        _ptr(floor), _ptr(den), _ptr(state), state.stride(0), _ptr(q_start), _ptr(positions), _ptr(state_slots), _ptr(o),
+        o.stride(0), entries, n, heads, dim, vdim, float(q_scale), int(bool(silu)), _stream()), "scalar_gate_scan")
+
+
+def diff_head_norm(a: torch.Tensor, lam: float, after: float, eps: float, gate: Optional[torch.Tensor], out: torch.Tensor,
+                   heads: int, vdim: int) -> None:
+    """Two attention maps over the same values combined head by head: ``a`` float32 ``[n, 2*heads*vdim]`` holds the
+    first map's heads, then the second's; ``out[:, h] = d / sqrt(mean(d^2) + eps) * after * sigmoid(gate[:, h])`` with
+    ``d = a1_h - lam a2_h`` (``gate`` float32 ``[n, heads]``, a column range of a wider matrix will do; ``None``: 1)."""
+    _f32_rows(a, "a")
+    _rows(out, "out", out.dtype)
+    n = a.shape[0]
+    _require(a.shape[1] == 2 * heads * vdim and out.shape == (n, heads * vdim), "a [n, 2*heads*vdim], out [n, heads*vdim]")
+    if gate is not None:
+        _f32_rows(gate, "gate")
+        _require(gate.shape == (n, heads), "gate must be [n, heads]")
+    _check(library().dli_diff_head_norm(_ptr(a), a.stride(0), float(lam), float(after), float(eps), _ptr(gate),
+                                        0 if gate is None else gate.stride(0), _ptr(out), out.stride(0), n, heads, vdim,
+                                        _is_bf16(out.dtype), _stream()), "diff_head_norm")
+
+
+def branch_weighted_sum(branches: Sequence[torch.Tensor], scales: Sequence[float], out: torch.Tensor) -> None:
+    """``out = sum_b scales[b] * branches[b]``: one to four float32 ``[n, width]`` matrices (rows contiguous)."""
+    _dense(out, "out", torch.float32, 2)
+    _require(1 <= len(branches) <= 4 and len(scales) == len(branches), "one to four branches, a scale each")
+    for i, y in enumerate(branches):
+        _f32_rows(y, f"branch {i}")
+        _require(y.shape == out.shape, "a branch differs from out in shape")
+    count = len(branches)
+    ptrs = (ctypes.c_void_p * count)(*[y.data_ptr() for y in branches])
+    strides = (ctypes.c_int64 * count)(*[y.stride(0) for y in branches])
+    sc = (ctypes.c_float * count)(*[float(x) for x in scales])
+    _check(library().dli_branch_weighted_sum(ptrs, strides, sc, count, _ptr(out), out.shape[0], out.shape[1], _stream()),
+           "branch_weighted_sum")
+
+
+def scale_f32(y: torch.Tensor, scale: float) -> None:
+    """``y *= scale`` in place (float32)."""
+    _dense(y, "y", torch.float32)
+    _check(library().dli_scale_f32(_ptr(y), y.numel(), float(scale), _stream()), "scale_f32")
+
+
+def table_choose(table: torch.Tensor, token_ids: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor) -> None:
+    """A router that is a table: ``ids[t] = table[token_ids[t]]`` (``table`` int32 ``[vocabulary, top]``), every
+    weight ``1 / top``."""
+    _dense(table, "table", torch.int32, 2)
+    _dense(token_ids, "token_ids", torch.int32, 1)
+    _dense(ids, "ids", torch.int32, 2)
+    _dense(weights, "weights", torch.float32, 2)
+    n, top = ids.shape
+    _require(table.shape[1] == top and token_ids.shape[0] == n and weights.shape == (n, top), "table, ids and weights disagree")
+    _check(library().dli_table_choose(_ptr(table), _ptr(token_ids), n, top, table.shape[0], _ptr(ids), _ptr(weights), _stream()),
+           "table_choose")

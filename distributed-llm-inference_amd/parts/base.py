@@ -46,7 +46,9 @@ class PagedKVSpec:
     ``window`` > 0: only the last ``window`` keys are ever read, so pages that lie wholly before
     the window may be given back while the request still runs. ``value_dim``: the size of a
     value where it differs from a key's (``None``: the same; 0: the mixer keeps keys only, a
-    compressed cache for instance, and gets no value pages). Layers with equal specs share one
+    compressed cache for instance, and gets no value pages). ``value_heads``: how many heads the value
+    pages hold where that is fewer than the keys' (``None``: as many; several key heads, the score maps
+    of one head for instance, then share a value head). Layers with equal specs share one
     group of pages and one block table.
     """
 
@@ -54,14 +56,21 @@ class PagedKVSpec:
     head_dim: int
     window: int = 0
     value_dim: Optional[int] = None
+    value_heads: Optional[int] = None
 
     def __post_init__(self) -> None:
         if self.kv_heads <= 0 or self.head_dim <= 0 or self.window < 0 or (self.value_dim or 0) < 0:
             raise ValueError(f"{self}: heads and sizes must be positive, window and value_dim not negative")
+        if self.value_heads is not None and (self.value_heads <= 0 or self.kv_heads % self.value_heads):
+            raise ValueError(f"{self}: the value heads must divide the kv heads")
 
     @property
     def v_dim(self) -> int:
         return self.head_dim if self.value_dim is None else self.value_dim
+
+    @property
+    def v_heads(self) -> int:
+        return self.kv_heads if self.value_heads is None else self.value_heads
 
 
 @dataclass(frozen=True)

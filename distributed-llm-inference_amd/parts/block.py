@@ -172,3 +172,44 @@ class PostNormBlock(Block):
             y = parts["feed_forward"].forward(h, ctx)
             parts["feed_forward_norm"].post_norm(x, y, self.alpha, ctx, gate=g, gate_bias=b)
         return x, None
+
+
+@register_part("block", "parallel_norms")
+class ParallelNormsBlock(Block):
+    """Mixer and feed-forward side by side, each behind a norm of its own, both reading the same stream:
+    ``x <- x + (mixer(norm1(x)) + feed_forward(norm2(x)))`` around a 32-bit residual stream. The feed-forward and
+    its norm may be absent. ``x`` is float32 in both runtimes; the norms round once, to the type that the
+    products read; the two results are added to each other and then into the stream, in 32-bit."""
+
+    roles = ("mixer_norm", "mixer")   # and, unless the layer has no feed-forward, "feed_forward_norm" and "feed_forward"
+
+    def __init__(self, runtime: Runtime) -> None:
+        super().__init__(runtime)
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on device arrays only
+
+    def forward(self, x: torch.Tensor, delta: Optional[torch.Tensor], ctx: Any, cache: Any,
+                parts: Mapping[str, Part]) -> tuple[torch.Tensor, Optional[torch.Tensor]]:
+        from ..kernels import ops
+
+        if x.dtype != torch.float32:
+            raise RuntimeError("the parallel_norms block keeps a float32 residual stream")
+        if delta is not None:
+            ops.add(x, delta, x)
+        y = _as_f32(parts["mixer"].forward(parts["mixer_norm"].forward(x), ctx, cache))
+        if "feed_forward" in parts:
+            f = _as_f32(parts["feed_forward"].forward(parts["feed_forward_norm"].forward(x), ctx))
+            ops.add(y, f, y)
+        ops.add(x, y, x)
+        return x, None
+
+
+def _as_f32(y: torch.Tensor) -> torch.Tensor:
+    if y.dtype == torch.float32:
+        return y
+    from ..kernels import ops
+
+    wide = torch.empty(y.shape, device=y.device, dtype=torch.float32)
+    ops.to_float(y, wide)
+    return wide

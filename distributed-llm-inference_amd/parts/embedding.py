@@ -9,20 +9,27 @@ import torch
 
 from ..kernels import ops
 from .base import DecodeStream, Embedding, Runtime
-from .registry import register_part
-from .spec import WeightSpec
+from .registry import build_part, register_part
+from .spec import PartSpec, WeightSpec
 
 
 @register_part("embedding", "token_embedding")
 class TokenEmbedding(Embedding):
     def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, weight_name: str = "weight",
-                 float32_rows: bool = False) -> None:
+                 float32_rows: bool = False, norm: Optional[PartSpec] = None) -> None:
         """``float32_rows``: the rows go out widened to float32 whatever the runtime's type, for a
-        model that keeps its residual stream in 32-bit (the table keeps the runtime's type)."""
+        model that keeps its residual stream in 32-bit (the table keeps the runtime's type). ``norm``: a norm
+        (a part with ``forward_f32``) that the float32 rows pass before they become the stream."""
         super().__init__(runtime)
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.weight_name, self.float32_rows = weight_name, bool(float32_rows)
         self.weight: torch.Tensor | None = None
+        if norm is not None and not self.float32_rows:
+            raise ValueError("a norm on the embedded rows belongs to a float32 stream")
+        self.norm = build_part("norm", norm, runtime) if norm is not None else None
+
+    def sub_parts(self) -> dict:
+        return {"norm": self.norm} if self.norm is not None else {}
 
     def graph_capturable(self, page_size: int) -> bool:
         return True  # kernels on device arrays only
@@ -49,7 +56,7 @@ class TokenEmbedding(Embedding):
             return self.forward(ctx.token_ids)
         out = torch.empty(ctx.token_ids.shape[0], self.hidden_size, device=self.rt.device, dtype=torch.float32)
         ops.embed_sinusoid(self.table(), ctx.token_ids, ctx.positions, None, out)
-        return out
+        return out if self.norm is None else self.norm.forward_f32(out)
 
     def streams(self, ctx) -> bool:
         return self.rt.is_bf16 and not self.float32_rows  # the fused decode kernels keep a stream of the runtime's type

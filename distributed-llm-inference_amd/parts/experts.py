@@ -15,6 +15,9 @@ limit, ``alpha = 1`` and ``up_shift = 0``: the plain ``silu(W_gate h) * (W_up h)
 expert of the same form (its own size and limit) may run for every token; it is added multiplied by
 ``sigmoid(W_sg h)``, one number per token, or as it is (``shared_gate=False``).
 
+``routing="table"``: no router; an integer tensor ``table [vocabulary, top]`` names each token id's experts (the
+entries of a row differ), each with the weight ``1 / top``.
+
 Order of work: one 32-bit product for the router (and the shared expert's gate: its row is stacked
 below the router's); the choice kernel; on the device the chosen (token, expert) pairs are sorted by
 expert and cut into row tiles, over which two kernels run the experts' products (nothing waits
@@ -40,8 +43,14 @@ class RoutedExperts(FeedForward):
     def __init__(self, runtime: Runtime, *, hidden_size: int, experts: int, top: int, expert_size: int,
                  limit: float, alpha: float = 1.702, identity: int = 0, groups: int = 1, groups_kept: int = 1,
                  scale: float = 1.0, correction: bool = True, shared_size: int = 0, shared_limit: float = 0.0,
-                 shared_gate: bool = True, up_shift: float = 1.0, router_bias: bool = False) -> None:
+                 shared_gate: bool = True, up_shift: float = 1.0, router_bias: bool = False, routing: str = "router",
+                 vocab_size: int = 0) -> None:
         super().__init__(runtime)
+        if routing not in ("router", "table"):
+            raise ValueError(f"routing must be 'router' or 'table', not {routing!r}")
+        if routing == "table" and (identity or vocab_size < 1 or shared_gate and shared_size):
+            raise ValueError("a table names real experts for every id of a vocabulary; a shared expert's gate needs a router")
+        self.routing, self.vocab_size, self.table = routing, int(vocab_size), None
         total = experts + identity
         if experts < 0 or identity < 0 or total < 1 or not 1 <= top <= min(total, 64):
             raise ValueError(f"{top} of {experts} experts and {identity} identity experts cannot be chosen")
@@ -63,10 +72,13 @@ class RoutedExperts(FeedForward):
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         h, f = self.hidden_size, self.expert_size
-        specs = {"router": WeightSpec((self.total, h))}
-        if self.has_router_bias:
+        if self.routing == "table":
+            specs = {"table": WeightSpec((self.vocab_size, self.top), role="int32", init=f"distinct_below:{self.experts}")}
+        else:
+            specs = {"router": WeightSpec((self.total, h))}
+        if self.routing == "router" and self.has_router_bias:
             specs["router.b"] = WeightSpec((self.total,), role="float32", init="zeros")
-        if self.has_correction:
+        if self.routing == "router" and self.has_correction:
             specs["correction"] = WeightSpec((self.total,), role="float32", init="zeros", optional=True)
         for e in range(self.experts):
             specs.update({f"e{e}.gate": WeightSpec((f, h)), f"e{e}.up": WeightSpec((f, h)), f"e{e}.down": WeightSpec((h, f))})
@@ -78,11 +90,16 @@ class RoutedExperts(FeedForward):
         return specs
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        rows = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_gate else [])
-        self.w_router = stack_rows(rows)
-        self.router_bias = tensors["router.b"].contiguous() if self.has_router_bias else None
-        # (a checkpoint without the tensor: scores are chosen as they are)
-        self.correction = tensors["correction"].contiguous() if self.has_correction and "correction" in tensors else None
+        if self.routing == "table":
+            self.table = tensors["table"].contiguous()
+            if self.table.numel() and not (0 <= int(self.table.min()) and int(self.table.max()) < self.experts):
+                raise ValueError(f"{self.prefix}table names experts outside 0..{self.experts - 1}")
+        else:
+            rows = [tensors["router"]] + ([tensors["shared.sg"]] if self.shared_gate else [])
+            self.w_router = stack_rows(rows)
+            self.router_bias = tensors["router.b"].contiguous() if self.has_router_bias else None
+            # (a checkpoint without the tensor: scores are chosen as they are)
+            self.correction = tensors["correction"].contiguous() if self.has_correction and "correction" in tensors else None
         if self.experts:
             self.w_gate = torch.stack([tensors[f"e{e}.gate"] for e in range(self.experts)]).contiguous()
             self.w_up = torch.stack([tensors[f"e{e}.up"] for e in range(self.experts)]).contiguous()
@@ -93,11 +110,15 @@ class RoutedExperts(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: Any) -> torch.Tensor:
         n, dev = x.shape[0], self.rt.device
-        logits = linear_f32(self.rt, x, self.w_router)
         ids = torch.empty(n, self.top, device=dev, dtype=torch.int32)
         weights = torch.empty(n, self.top, device=dev, dtype=torch.float32)
-        ops.router_choose(logits, self.total, self.correction, self.groups, self.groups_kept, self.top, self.scale, ids, weights,
-                          bias=self.router_bias)
+        if self.routing == "table":
+            logits = None
+            ops.table_choose(self.table, ctx.token_ids, ids, weights)
+        else:
+            logits = linear_f32(self.rt, x, self.w_router)
+            ops.router_choose(logits, self.total, self.correction, self.groups, self.groups_kept, self.top, self.scale, ids,
+                              weights, bias=self.router_bias)
         z = None
         if self.experts:
             z = ops.expert_products(ids, x, self.w_gate, self.w_up, self.w_down, self.limit, self.alpha, self.up_shift)

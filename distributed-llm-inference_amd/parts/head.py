@@ -17,10 +17,11 @@ from .spec import WeightSpec
 @register_part("head", "linear_head")
 class LinearHead(Head):
     def __init__(self, runtime: Runtime, *, vocab_size: int, hidden_size: int, tied: bool,
-                 softcap: float = 0.0) -> None:
+                 softcap: float = 0.0, scale: float = 1.0) -> None:
         super().__init__(runtime)
         self.vocab_size, self.hidden_size, self.tied = vocab_size, hidden_size, tied
         self.softcap = float(softcap)  # > 0: logits <- softcap * tanh(logits / softcap)
+        self.scale = float(scale)      # the logits are multiplied by it (before a soft cap)
         self.weight: Optional[torch.Tensor] = None
         self.weight_tiled: Optional[torch.Tensor] = None
 
@@ -45,6 +46,8 @@ class LinearHead(Head):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         logits = self._logits(x)
+        if self.scale != 1.0:
+            ops.scale_f32(logits, self.scale)
         if self.softcap > 0:
             ops.softcap(logits, self.softcap)
         return logits
@@ -70,7 +73,7 @@ class LinearHead(Head):
         return out
 
     def streams(self, ctx) -> bool:
-        return self.softcap == 0 and self.rt.is_bf16 and (ctx.num_tokens > self.FEW_ROWS
+        return self.softcap == 0 and self.scale == 1.0 and self.rt.is_bf16 and (ctx.num_tokens > self.FEW_ROWS
                                     or ops.skinny_gemm_supports(ctx.num_tokens, self.hidden_size, self.rt.dtype))
 
     def forward_stream(self, stream: DecodeStream, norm: Norm, argmax: Optional[ArgmaxStage] = None) -> torch.Tensor:

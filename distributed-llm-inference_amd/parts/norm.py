@@ -15,19 +15,29 @@ from .spec import WeightSpec
 
 @register_part("norm", "rms_norm")
 class RMSNorm(Norm):
-    def __init__(self, runtime: Runtime, *, width: int, eps: float, weight_name: str = "weight") -> None:
+    def __init__(self, runtime: Runtime, *, width: int, eps: float, weight_name: str = "weight",
+                 unit_offset: bool = False) -> None:
+        """``unit_offset``: the checkpoint stores the weight around zero and the norm multiplies by one plus it
+        (the sum is made once, at load, in 32-bit; every kernel then sees an ordinary weight)."""
         super().__init__(runtime)
-        self.width, self.eps, self.weight_name = width, float(eps), weight_name
+        self.width, self.eps, self.weight_name, self.unit_offset = width, float(eps), weight_name, bool(unit_offset)
         self.weight: torch.Tensor | None = None
 
     def graph_capturable(self, page_size: int) -> bool:
         return True  # kernels on device arrays only
 
     def weight_specs(self) -> dict[str, WeightSpec]:
-        return {self.weight_name: WeightSpec((self.width,), role="float32", init="norm")}
+        return {self.weight_name: WeightSpec((self.width,), role="float32", init="zeros" if self.unit_offset else "norm")}
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.weight_name]
+        w = tensors[self.weight_name]
+        self.weight = (w + 1.0).contiguous() if self.unit_offset else w
+
+    def forward_f32(self, x: torch.Tensor) -> torch.Tensor:
+        """The norm of a float32 ``x`` as float32 whatever the runtime's type (a norm inside a 32-bit stream)."""
+        out = torch.empty_like(x)
+        ops.rms_norm_from_f32(x, self.weight, self.eps, out)
+        return out
 
     def fused_params(self) -> tuple[torch.Tensor, float]:
         """Weight and eps, for a consumer that computes this norm inside its own kernel."""

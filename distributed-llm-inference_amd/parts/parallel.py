@@ -1,6 +1,7 @@
 """Mixers side by side: every branch reads the same rows, each branch's output is divided by its
 root mean square over the model width and multiplied by a weight of its own (a plain weight, not
-one plus it), and the result is the mean of the branches.
+one plus it), and the result is the mean of the branches (``combine="norm_mean"``); or the result is
+the sum of the branches' outputs, each times a constant of its own (``combine="weighted_sum"``, ``scales``).
 
 The branches are mixers of any kind, given as part specs with their own tensor prefixes; each keeps
 whatever it keeps per request (pages, a state, nothing), and the pair's cache is the composite of
@@ -28,13 +29,23 @@ from .spec import PartSpec, WeightSpec
 class ParallelMixers(Mixer):
     MAX_BRANCHES = 4  # what the kernel that normalises and averages takes
 
+    COMBINE = ("norm_mean", "weighted_sum")
+
     def __init__(self, runtime: Runtime, *, hidden_size: int, branches: Mapping[str, PartSpec], norm_eps: float = 1e-6,
-                 out_weight_names: Optional[Mapping[str, str]] = None) -> None:
+                 out_weight_names: Optional[Mapping[str, str]] = None, combine: str = "norm_mean",
+                 scales: Optional[Mapping[str, float]] = None) -> None:
         """``branches``: name -> the branch's mixer. ``out_weight_names``: name -> the tensor (below
-        this part's prefix) that multiplies the branch's normalised output; default ``<name>.out``."""
+        this part's prefix) that multiplies the branch's normalised output; default ``<name>.out``.
+        ``combine="weighted_sum"``: no norms and no tensors, ``scales``: name -> the branch's constant."""
         super().__init__(runtime)
         if not 1 <= len(branches) <= self.MAX_BRANCHES:
             raise ValueError(f"one to {self.MAX_BRANCHES} branches, not {len(branches)}")
+        if combine not in self.COMBINE:
+            raise ValueError(f"combine must be one of {self.COMBINE}")
+        if combine == "weighted_sum" and set(scales or {}) != set(branches):
+            raise ValueError("a weighted sum needs a scale for every branch")
+        self.combine = combine
+        self.scales = {n: float(v) for n, v in (scales or {}).items()}
         self.hidden_size, self.norm_eps = hidden_size, float(norm_eps)
         self.names = list(branches)
         self.branches = {name: build_part("mixer", spec, runtime) for name, spec in branches.items()}
@@ -47,6 +58,8 @@ class ParallelMixers(Mixer):
         return dict(self.branches)
 
     def weight_specs(self) -> dict[str, WeightSpec]:
+        if self.combine == "weighted_sum":
+            return {}
         return {self.out_names[n]: WeightSpec((self.hidden_size,), role="float32", init="norm") for n in self.names}
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
@@ -89,5 +102,8 @@ class ParallelMixers(Mixer):
                 y = wide
             outs.append(y)
         out = torch.empty(x.shape[0], self.hidden_size, device=self.rt.device, dtype=torch.float32)
-        ops.branch_norm_mean(outs, [self.out_w[n] for n in self.names], self.norm_eps, out)
+        if self.combine == "weighted_sum":
+            ops.branch_weighted_sum(outs, [self.scales[n] for n in self.names], out)
+        else:
+            ops.branch_norm_mean(outs, [self.out_w[n] for n in self.names], self.norm_eps, out)
         return out

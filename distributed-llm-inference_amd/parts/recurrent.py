@@ -1,11 +1,12 @@
 """Mixers that carry a matrix state per head from token to token instead of a cache of keys:
 ``general_delta`` (a generalized delta rule), ``wkv`` (decayed sums with a bonus for the current
 token and token shift), ``gated_delta`` (the delta rule with one decay and one write strength per
-head, behind short convolutions) and ``gated_linear`` (decayed sums whose forget gate also decides what
-is written). The state lives in 32-bit in the request's state slot
+head, behind short convolutions), ``gated_linear`` (decayed sums whose forget gate also decides what
+is written), ``matrix_memory`` (exponential input and forget gates, one pair a head, with a normaliser) and
+``decayed_linear`` (linear attention with a constant decay per head). The state lives in 32-bit in the request's state slot
 (:class:`StateSpec`), starts at zero at position 0, and is all that a step leaves for the next.
 
-Both run their projections as products of the runtime's type with 32-bit sums, and everything
+All run their projections as products of the runtime's type with 32-bit sums, and everything
 after them in 32-bit: decays, rates, unit keys, the recurrence, the per-head norm of its output
 and the gate (``csrc/recurrent_scan.hip``). The decay's pre-activation is a low-rank projection,
 ``W2 tanh(W1 h) + w0``, whose second half is 32-bit; its rank is read off the checkpoint's tensor.
@@ -294,4 +295,143 @@ class GatedLinear(Mixer):
                               self.num_heads, self.head_dim, self.value_dim)
         out = self.rt.empty(n, self.hv)
         ops.head_norm_gate(o, None, self.norm_w, self.norm_eps, out, self.num_heads, self.value_dim, gate="none")
+        return linear_f32(self.rt, out, self.w_o)
+
+
+class _ScalarGateMixer(Mixer):
+    """What the recurrences under scalar gates share: ``S <- a S + b k v^T``, ``o = S^T q`` per head with one keep
+    factor ``a`` and one write factor ``b`` a token and head (``csrc/scalar_gate_scan.hip``)."""
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, head_dim: int, value_dim: Optional[int] = None,
+                 norm_eps: float = 1e-6) -> None:
+        super().__init__(runtime)
+        value_dim = head_dim if value_dim is None else value_dim
+        if min(hidden_size, num_heads, head_dim, value_dim) < 1:
+            raise ValueError("heads and their sizes must be positive")
+        self.hidden_size, self.num_heads, self.head_dim, self.value_dim = hidden_size, num_heads, head_dim, value_dim
+        self.norm_eps = float(norm_eps)
+        self.hd, self.hv = num_heads * head_dim, num_heads * value_dim
+        self.w_in = self.norm_w = self.w_o = None
+
+    def graph_capturable(self, page_size: int) -> bool:
+        return True  # kernels on the context's device arrays only; padding rows write the spare slot
+
+    def input_weight(self) -> Optional[torch.Tensor]:
+        """The matrix of the one product that reads the rows, for whoever stacks it with others'
+        (``forward`` then gets the product's result as ``proj``)."""
+        return self.w_in
+
+    def release_input_weight(self) -> None:
+        self.w_in = None
+
+    def _state(self, cache: Any) -> torch.Tensor:
+        if cache is None or cache.kind != "state" or not cache.writable:
+            raise RuntimeError(f"{self.kind} needs a state of its own")
+        return cache.state.view(cache.state.shape[0], -1)
+
+
+@register_part("mixer", "matrix_memory")
+class MatrixMemory(_ScalarGateMixer):
+    """A matrix memory with exponential gates. From the rows ``h``: ``q = W_q h * head_dim^-1/2`` and ``k = W_k h``
+    (``num_heads x head_dim``), ``v = W_v h`` (``num_heads x value_dim``), and per head the log input gate
+    ``i = cap tanh((W_i h + b_i) / cap)`` and the log forget gate ``f = logsigmoid(cap tanh((W_f h + b_f) / cap))``
+    (``gate_cap`` 0: no cap). With a running reference point ``m`` that starts at 0 (not at minus infinity):
+    ``m' = max(f + m, i)``, ``S' = e^(f + m - m') S + e^(i - m') k v^T``, ``n'`` alike from ``k`` alone, and
+    ``o = S'^T q / (max(|n' . q|, e^(-m')) + 1e-6)``. Each head's ``o`` is divided by its root mean square, the heads
+    side by side are multiplied by ``norm`` (all heads' size) and by ``sigmoid(W_g h)``, then the output product.
+    The request's state slot holds ``S`` with ``n`` as one more column a head, then ``m``, all 32-bit; everything
+    between the projections and the output product is 32-bit."""
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, head_dim: int, value_dim: Optional[int] = None,
+                 norm_eps: float = 1e-6, gate_cap: float = 0.0) -> None:
+        super().__init__(runtime, hidden_size=hidden_size, num_heads=num_heads, head_dim=head_dim, value_dim=value_dim,
+                         norm_eps=norm_eps)
+        if gate_cap < 0:
+            raise ValueError("the gates' cap must not be negative")
+        self.gate_cap = float(gate_cap)
+        self.state_floats = num_heads * (self.value_dim + 1) * head_dim
+        self.i_bias = self.f_bias = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h, H = self.hidden_size, self.num_heads
+        return {"q": WeightSpec((self.hd, h)), "k": WeightSpec((self.hd, h)), "v": WeightSpec((self.hv, h)),
+                "g": WeightSpec((self.hv, h)), "i": WeightSpec((H, h)), "f": WeightSpec((H, h)),
+                "i.b": WeightSpec((H,), role="float32", init="zeros"), "f.b": WeightSpec((H,), role="float32", init="zeros"),
+                "norm": WeightSpec((self.hv,), role="float32", init="norm"), "o": WeightSpec((h, self.hv))}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_in = stack_rows([tensors[n] for n in ("q", "k", "v", "g", "i", "f")])   # one product for everything that reads h
+        self.i_bias, self.f_bias = tensors["i.b"].contiguous(), tensors["f.b"].contiguous()
+        self.norm_w, self.w_o = tensors["norm"].contiguous(), tensors["o"]
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.state_floats + self.num_heads,), torch.float32)
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+        state = self._state(cache)
+        n, H = x.shape[0], self.num_heads
+        if proj is None:
+            proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
+        k0, v0, g0 = self.hd, 2 * self.hd, 2 * self.hd + self.hv
+        i0 = g0 + self.hv
+        keep, write, floor = ops.exp_gates(proj, i0, i0 + H, self.i_bias, self.f_bias, self.gate_cap, state, self.state_floats,
+                                           ctx.q_start, ctx.positions, ctx.state_slots, H)
+        o = torch.empty(n, self.hv, device=self.rt.device, dtype=torch.float32)
+        den = torch.empty(n, H, device=self.rt.device, dtype=torch.float32)
+        ops.scalar_gate_scan(proj[:, :k0], proj[:, k0:v0], proj[:, v0:g0], state, ctx.q_start, ctx.positions, ctx.state_slots,
+                             o, H, self.head_dim, self.value_dim, keep=keep, write=write, floor=floor, den=den,
+                             q_scale=self.head_dim ** -0.5)
+        out = self.rt.empty(n, self.hv)
+        ops.head_norm_gate(o, proj[:, g0:g0 + self.hv], self.norm_w, self.norm_eps, out, H, self.value_dim, gate="sigmoid",
+                           den=den)
+        return linear_f32(self.rt, out, self.w_o)
+
+
+@register_part("mixer", "decayed_linear")
+class DecayedLinear(_ScalarGateMixer):
+    """Linear attention with a constant decay per head. From the rows ``h``: ``q = silu(W_q h)`` and
+    ``k = silu(W_k h)`` (``num_heads x head_dim``), ``v = silu(W_v h)`` (``num_heads x value_dim``); per head
+    ``S <- decay S + k v^T``, ``o = S^T q`` (no other scale). The heads side by side are divided by their root mean
+    square over all of them, multiplied by ``norm`` and by ``sigmoid(W_g h)``, then the output product. The
+    request's state slot holds ``S`` in 32-bit; everything between the projections and the output product is 32-bit."""
+
+    def __init__(self, runtime: Runtime, *, hidden_size: int, num_heads: int, head_dim: int, decay: Any,
+                 value_dim: Optional[int] = None, norm_eps: float = 1e-6) -> None:
+        super().__init__(runtime, hidden_size=hidden_size, num_heads=num_heads, head_dim=head_dim, value_dim=value_dim,
+                         norm_eps=norm_eps)
+        self.decay_values = [float(d) for d in decay]
+        if len(self.decay_values) != num_heads:
+            raise ValueError(f"{len(self.decay_values)} decays for {num_heads} heads")
+        self.decay: Optional[torch.Tensor] = None
+
+    def weight_specs(self) -> dict[str, WeightSpec]:
+        h = self.hidden_size
+        return {"q": WeightSpec((self.hd, h)), "k": WeightSpec((self.hd, h)), "v": WeightSpec((self.hv, h)),
+                "g": WeightSpec((self.hv, h)), "norm": WeightSpec((self.hv,), role="float32", init="norm"),
+                "o": WeightSpec((h, self.hv))}
+
+    def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
+        self.w_in = stack_rows([tensors[n] for n in ("q", "k", "v", "g")])   # one product for everything that reads h
+        self.norm_w, self.w_o = tensors["norm"].contiguous(), tensors["o"]
+
+    def finalize(self) -> None:
+        self.decay = torch.tensor(self.decay_values, dtype=torch.float32, device=self.rt.device)
+
+    def cache_spec(self) -> StateSpec:
+        return StateSpec((self.num_heads * self.value_dim * self.head_dim,), torch.float32)
+
+    def forward(self, x: torch.Tensor, ctx: Any, cache: Any, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
+        state = self._state(cache)
+        n = x.shape[0]
+        if proj is None:
+            proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
+        if self.decay is None:
+            self.finalize()
+        k0, v0, g0 = self.hd, 2 * self.hd, 2 * self.hd + self.hv
+        o = torch.empty(n, self.hv, device=self.rt.device, dtype=torch.float32)
+        ops.scalar_gate_scan(proj[:, :k0], proj[:, k0:v0], proj[:, v0:g0], state, ctx.q_start, ctx.positions, ctx.state_slots,
+                             o, self.num_heads, self.head_dim, self.value_dim, decay=self.decay, silu=True)
+        out = self.rt.empty(n, self.hv)
+        # one norm over all heads: the row as a single head
+        ops.head_norm_gate(o, proj[:, g0:g0 + self.hv], self.norm_w, self.norm_eps, out, 1, self.hv, gate="sigmoid")
         return linear_f32(self.rt, out, self.w_o)

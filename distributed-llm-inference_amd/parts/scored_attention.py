@@ -1,6 +1,8 @@
 """Grouped-query attention over the paged cache whose scores are changed by parameters: unit-RMS
 queries and keys or a rotary position encoding, a per-head logarithmic distance penalty, a chunked
-mask, a softmax with a sink, value mixing across layers, and a sigmoid output gate. Each is a
+mask, a window that keeps the first positions, a softmax with a sink, value mixing across layers, a sigmoid
+output gate, biases on the projections, several score maps a head over the same values whose results are
+subtracted (differential attention), and keys and values read from another layer's cache. Each is a
 parameter, so another design may take any subset.
 
 Order of work for the rows ``h`` of a step (``x`` may be a 32-bit residual stream; the products read
@@ -19,6 +21,15 @@ it in the runtime's type):
    ``exp(s_ij) / (sink + sum_j exp(s_ij))`` with ``sink = 1`` (a key of score 0 that has no value),
    the result multiplied by ``sigmoid(gate)``;
 4. the output product, 32-bit sums.
+
+With ``maps=2`` every query head and every kv head has two sets of ``head_dim`` components (the checkpoint lays
+them out head by head as map 1, map 2; they are reordered at load to all heads' first maps, then all second
+maps, so that each map is a head of its own to the kernels, and the value pages hold one head per kv head
+that both maps read). Each map is a softmax attention of its own; with ``a1, a2`` their results and
+``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff`` (four vectors of ``head_dim`` values, one number a layer),
+the head's result is ``d / sqrt(mean(d^2) + norm_eps) * (1 - diff)`` with ``d = a1 - lambda a2``, times
+``sigmoid(W_g h)_head`` where ``head_gate`` (one number a head). ``own_kv=False``: the layer has no key and value
+projections and reads the cache of the schedule entry it is given (keys as that layer rotated them).
 
 Scores, weights, norms and the mixing are 32-bit; keys and values are cached in the runtime's type.
 """
@@ -74,8 +85,23 @@ class ScoredAttention(Mixer):
                  norm_eps: float = 1e-6, distance_penalty: bool = False, chunk: int = 0, window: int = 0,
                  sink: bool = False, output_gate: bool = False, value_mix: str = "none",
                  value_mix_key: str = "first_values", names: Optional[Mapping[str, str]] = None,
-                 position: Optional[PartSpec] = None) -> None:
+                 position: Optional[PartSpec] = None, bias: bool = False, keep_first: int = 0, maps: int = 1,
+                 diff: float = 0.0, head_gate: bool = False, own_kv: bool = True) -> None:
         super().__init__(runtime)
+        if maps not in (1, 2):
+            raise ValueError("one score map a head, or two whose results are subtracted")
+        if maps == 2 and (qk_unit or output_gate or value_mix != "none"):
+            raise ValueError("scored_attention: two maps a head go with rotary or plain keys and a gate per head")
+        if head_gate and maps != 2:
+            raise ValueError("scored_attention: the gate per head belongs to the kernel that combines two maps")
+        if (bias or not own_kv) and qk_unit:
+            raise ValueError("scored_attention: biases and borrowed keys go with rotary or plain keys")
+        if keep_first < 0 or (keep_first and not window):
+            raise ValueError("scored_attention: kept first positions belong to a window")
+        self.bias, self.keep_first, self.maps, self.diff = bool(bias), int(keep_first), int(maps), float(diff)
+        self.head_gate, self.own_kv = bool(head_gate), bool(own_kv)
+        self.b_in = None
+        self.lam = 0.0
         if num_heads < 1 or num_kv_heads < 1 or num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads do not group onto {num_kv_heads} kv heads")
         value_dim = head_dim if value_dim is None else value_dim
@@ -98,21 +124,21 @@ class ScoredAttention(Mixer):
         if not self.qk_unit and value_mix != "none":
             raise ValueError("scored_attention: value mixing belongs to the kernel that makes unit keys")
         self.names = {"q": "q", "k": "k", "v": "v", "g": "g", "o": "o", "mix": "vmix", "r1": "r1", "r2": "r2",
-                      **dict(names or {})}
+                      "lq1": "lq1", "lk1": "lk1", "lq2": "lq2", "lk2": "lk2", **dict(names or {})}
         self.w_in = self.w_o = self.mix = self.r1 = self.r2 = None
 
     # -- sizes of the stacked projection's parts
     @property
     def _q(self) -> int:
-        return self.num_heads * self.head_dim
+        return self.num_heads * self.maps * self.head_dim
 
     @property
     def _k(self) -> int:
-        return self.num_kv_heads * self.head_dim
+        return self.num_kv_heads * self.maps * self.head_dim if self.own_kv else 0
 
     @property
     def _v(self) -> int:
-        return self.num_kv_heads * self.value_dim
+        return self.num_kv_heads * self.value_dim if self.own_kv else 0
 
     @property
     def _o(self) -> int:
@@ -120,10 +146,18 @@ class ScoredAttention(Mixer):
 
     def weight_specs(self) -> dict[str, WeightSpec]:
         n, h = self.names, self.hidden_size
-        specs = {n["q"]: WeightSpec((self._q, h)), n["k"]: WeightSpec((self._k, h)), n["v"]: WeightSpec((self._v, h)),
-                 n["o"]: WeightSpec((h, self._o))}
+        specs = {n["q"]: WeightSpec((self._q, h)), n["o"]: WeightSpec((h, self._o))}
+        if self.own_kv:
+            specs.update({n["k"]: WeightSpec((self._k, h)), n["v"]: WeightSpec((self._v, h))})
+        if self.bias:
+            specs.update({n[s] + ".b": WeightSpec((size,), role="float32", init="zeros")
+                          for s, size in (("q", self._q), ("k", self._k), ("v", self._v)) if size})
         if self.output_gate:
             specs[n["g"]] = WeightSpec((self._o, h))
+        if self.head_gate:
+            specs[n["g"]] = WeightSpec((self.num_heads, h))
+        if self.maps == 2:
+            specs.update({n[s]: WeightSpec((self.head_dim,), role="float32", init="zeros") for s in ("lq1", "lk1", "lq2", "lk2")})
         if self.distance_penalty:
             specs[n["r1"]] = WeightSpec((self.num_heads,), role="float32", init="norm")
             specs[n["r2"]] = WeightSpec((self.num_heads,), role="float32", init="norm")
@@ -134,8 +168,24 @@ class ScoredAttention(Mixer):
 
     def load_weights(self, tensors: Mapping[str, torch.Tensor]) -> None:
         n = self.names
-        stacked = [tensors[n["q"]], tensors[n["k"]], tensors[n["v"]]] + ([tensors[n["g"]]] if self.output_gate else [])
+
+        def by_map(t: torch.Tensor, heads: int) -> torch.Tensor:
+            """Rows (or entries) laid out head by head as [map 1, map 2] become all first maps, then all second."""
+            if self.maps == 1:
+                return t
+            return t.reshape(heads, self.maps, self.head_dim, *t.shape[1:]).transpose(0, 1).reshape(t.shape)
+
+        kinds = [("q", self.num_heads)] + ([("k", self.num_kv_heads), ("v", 0)] if self.own_kv else [])
+        stacked = [by_map(tensors[n[s]], heads) if heads else tensors[n[s]] for s, heads in kinds]
+        if self.output_gate or self.head_gate:
+            stacked.append(tensors[n["g"]])
         self.w_in = stack_rows(stacked)
+        if self.bias:
+            b = torch.cat([by_map(tensors[n[s] + ".b"], heads) if heads else tensors[n[s] + ".b"] for s, heads in kinds])
+            self.b_in = torch.cat([b, b.new_zeros(self.w_in.shape[0] - b.shape[0])]).contiguous()
+        if self.maps == 2:
+            lq1, lk1, lq2, lk2 = (tensors[n[s]].float() for s in ("lq1", "lk1", "lq2", "lk2"))
+            self.lam = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum())) + self.diff
         self.w_o = tensors[n["o"]]
         if self.distance_penalty:
             self.r1, self.r2 = tensors[n["r1"]].contiguous(), tensors[n["r2"]].contiguous()
@@ -153,9 +203,13 @@ class ScoredAttention(Mixer):
         if table is None and type(self.position).apply is not PositionEncoding.apply:
             raise ops.KernelArgumentError("scored_attention takes a rotary table or no position encoding")
 
-    def cache_spec(self) -> PagedKVSpec:
-        return PagedKVSpec(self.num_kv_heads, self.head_dim, self.window,
-                           None if self.value_dim == self.head_dim else self.value_dim)
+    def cache_spec(self) -> Optional[PagedKVSpec]:
+        if not self.own_kv:
+            return None   # the schedule hands this layer another entry's cache
+        # (a window that keeps its first positions gives no page back while the request runs)
+        return PagedKVSpec(self.num_kv_heads * self.maps, self.head_dim, 0 if self.keep_first else self.window,
+                           None if self.value_dim == self.head_dim else self.value_dim,
+                           self.num_kv_heads if self.maps > 1 else None)
 
     def graph_capturable(self, page_size: int) -> bool:
         return True  # a step of single tokens is read through the context's device arrays alone
@@ -169,8 +223,8 @@ class ScoredAttention(Mixer):
         self.w_in = None
 
     def forward(self, x: torch.Tensor, ctx: Any, cache: Any, proj: Optional[torch.Tensor] = None) -> torch.Tensor:
-        if cache is None or cache.kind != "paged" or not cache.writable:
-            raise RuntimeError("scored_attention needs a paged cache of its own")
+        if cache is None or cache.kind != "paged" or cache.writable != self.own_kv:
+            raise RuntimeError("scored_attention needs a paged cache: its own, or with own_kv=False another entry's")
         grp = ctx.groups[cache.group]
         n = x.shape[0]
         if proj is None:
@@ -192,10 +246,22 @@ class ScoredAttention(Mixer):
             table = self.position.rotary_table()
             ops.rotary_cache(proj, 0, self._q, self._q + self._k, ctx.positions, None if table is None else table.inv_freq,
                              0 if table is None else table.dim, table is not None and table.pairing == "interleaved",
-                             q, grp.slots, cache.k_pages, cache.v_pages, self.num_heads)
-        out = self.rt.empty(n, self._o)
+                             q, grp.slots if self.own_kv else None, cache.k_pages if self.own_kv else None,
+                             cache.v_pages if self.own_kv else None, self.num_heads * self.maps, bias=self.b_in)
         g0 = self._q + self._k + self._v
+        if self.maps == 2:
+            # each map is a head of its own to the attention kernels; their results stay 32-bit until they are combined
+            both = torch.empty(n, 2 * self._o, device=self.rt.device, dtype=torch.float32)
+            paged_scored_attention(self.rt, ctx, cache, q, both, 2 * self.num_heads, self.head_dim, self.value_dim, self.scale,
+                                   window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2,
+                                   keep_first=self.keep_first)
+            out = self.rt.empty(n, self._o)
+            ops.diff_head_norm(both, self.lam, 1.0 - self.diff, self.norm_eps,
+                               proj[:, g0:g0 + self.num_heads] if self.head_gate else None, out, self.num_heads, self.value_dim)
+            return linear_f32(self.rt, out, self.w_o)
+        out = self.rt.empty(n, self._o)
         gate = proj[:, g0:g0 + self._o] if self.output_gate else None
         paged_scored_attention(self.rt, ctx, cache, q, out, self.num_heads, self.head_dim, self.value_dim, self.scale,
-                               gate=gate, window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2)
+                               gate=gate, window=self.window, chunk=self.chunk, sink=self.sink, r1=self.r1, r2=self.r2,
+                               keep_first=self.keep_first)
         return linear_f32(self.rt, out, self.w_o)

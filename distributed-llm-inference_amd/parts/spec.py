@@ -27,7 +27,8 @@ class WeightSpec:
     shape: tuple[int, ...]
     role: str = "matrix"
     optional: bool = False
-    init: str = "normal"  # random-weights mode: "normal" (std 0.02), "ones", "zeros", "norm"
+    init: str = "normal"  # random-weights mode: "normal" (std 0.02), "ones", "zeros", "norm"; an integer table:
+    #                       "distinct_below:<n>" (every row different numbers below n), else zeros
     # A size that only the checkpoint gives is -1 in ``shape`` (any size fits; the part reads it off
     # the tensor it receives); ``drawn_shape`` is then the shape that random-weights mode draws.
     drawn_shape: Optional[tuple[int, ...]] = None

@@ -82,7 +82,13 @@ def write_random_model(out_dir: str | Path, config: Mapping[str, Any] | Any, *, 
     tensors: dict[str, tuple[str, np.ndarray]] = {}
     for name, spec in model.weight_specs().items():
         if spec.role == "int32":
-            tensors[name] = ("I32", np.zeros(spec.shape_to_draw, np.int32))
+            table = np.zeros(spec.shape_to_draw, np.int32)
+            if spec.init.startswith("distinct_below:") and table.ndim == 2:
+                # every row holds different numbers below the bound (a table of choices)
+                bound = int(spec.init.split(":", 1)[1])
+                keys = _generator(seed, name).random((table.shape[0], bound))
+                table = np.argsort(keys, axis=1)[:, :table.shape[1]].astype(np.int32)
+            tensors[name] = ("I32", table)
             continue
         if torch.device(device).type != "cpu":
             t = _drawn_on_device(name, spec.shape_to_draw, spec.init, seed, std, norm_jitter, torch.device(device))
