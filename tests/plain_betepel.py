@@ -102,6 +102,13 @@ def masked_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, first: i
     return out
 
 
+def attention_sizes(m: Mapping[str, Any]) -> tuple:
+    """heads, kv heads (absent: as many), key size, value size (absent: the key's), scale (absent: dim^-1/2)."""
+    H, d = m["heads"], m["dim"]
+    scale = m.get("scale")
+    return H, m.get("kv_heads") or H, d, m.get("vdim") or d, float(scale) if scale is not None else d ** -0.5
+
+
 def project(h: torch.Tensor, p: Mapping[str, torch.Tensor], name: str) -> torch.Tensor:
     y = h @ p[name].t()
     return y + p[name + ".b"] if name + ".b" in p else y
@@ -110,7 +117,8 @@ def project(h: torch.Tensor, p: Mapping[str, torch.Tensor], name: str) -> torch.
 def keys_values(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Mapping[str, Any], maps: int, first: int,
                 state: dict) -> tuple:
     """This call's rotated keys and values appended to what ``state`` holds; keys ``[total, kv * maps, d]``."""
-    n, G, d, dv = h.shape[0], m["kv_heads"], m["dim"], m["vdim"]
+    n = h.shape[0]
+    _, G, d, dv, _ = attention_sizes(m)
     pos = torch.arange(first, first + n)
     k = rotate(project(h, p, "k").view(n, G * maps, d), pos, m.get("rot"))
     v = project(h, p, "v").view(n, G, dv)
@@ -125,7 +133,8 @@ def differential_attention(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Ma
     """Two score maps per head over the same values: ``o = a1 - lam a2``, normalised per head without a
     weight, times ``1 - diff``, times one gate per head. ``borrowed``: another layer's state with keys and
     values (this layer then has none of its own)."""
-    n, H, G, d, dv = h.shape[0], m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    n = h.shape[0]
+    H, G, d, dv, scale = attention_sizes(m)
     pos = torch.arange(first, first + n)
     q = rotate(project(h, p, "q").view(n, H * 2, d), pos, m.get("rot")).view(n, H, 2, d)
     if borrowed is None:
@@ -133,8 +142,8 @@ def differential_attention(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Ma
     else:
         k, v = borrowed["k"], borrowed["v"]
     k = k.view(-1, G, 2, d)
-    a1 = masked_attention(q[:, :, 0], k[:, :, 0], v, first, m["scale"], m.get("mask"))
-    a2 = masked_attention(q[:, :, 1], k[:, :, 1], v, first, m["scale"], m.get("mask"))
+    a1 = masked_attention(q[:, :, 0], k[:, :, 0], v, first, scale, m.get("mask"))
+    a2 = masked_attention(q[:, :, 1], k[:, :, 1], v, first, scale, m.get("mask"))
     diff = float(m["diff"])
     lam = torch.exp((p["lq1"] * p["lk1"]).sum()) - torch.exp((p["lq2"] * p["lk2"]).sum()) + diff
     o = rms(a1 - lam * a2, eps) * (1.0 - diff)
@@ -144,11 +153,12 @@ def differential_attention(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Ma
 
 def windowed_attention(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Mapping[str, Any], first: int,
                        state: dict) -> torch.Tensor:
-    n, H, d = h.shape[0], m["heads"], m["dim"]
+    n = h.shape[0]
+    H, _, d, _, scale = attention_sizes(m)
     pos = torch.arange(first, first + n)
     q = rotate(project(h, p, "q").view(n, H, d), pos, m.get("rot"))
     k, v = keys_values(h, p, m, 1, first, state)
-    o = masked_attention(q, k, v, first, m["scale"], m.get("mask"))
+    o = masked_attention(q, k, v, first, scale, m.get("mask"))
     return o.reshape(n, -1) @ p["o"].t()
 
 
@@ -166,7 +176,8 @@ def decayed_linear_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
 
 
 def lightning(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Mapping[str, Any], eps: float, state: dict) -> torch.Tensor:
-    n, H, d, dv = h.shape[0], m["heads"], m["dim"], m["vdim"]
+    n, H, d = h.shape[0], m["heads"], m["dim"]
+    dv = m.get("vdim") or d
     q, k = silu(h @ p["q"].t()).view(n, H, d), silu(h @ p["k"].t()).view(n, H, d)
     v = silu(h @ p["v"].t()).view(n, H, dv)
     o, state["S"] = decayed_linear_attention(q, k, v, torch.tensor(m["decay"], dtype=F), state.get("S"))
@@ -178,7 +189,7 @@ def side_by_side(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Mapping[str,
                  state: dict) -> torch.Tensor:
     left = windowed_attention(h, sub_tensors(p, "left."), m["left"], first, state.setdefault("left", {}))
     right = lightning(h, sub_tensors(p, "right."), m["right"], eps, state.setdefault("right", {}))
-    return float(m["left_scale"]) * left + float(m["right_scale"]) * right
+    return float(m.get("left_scale", 1.0)) * left + float(m.get("right_scale", 1.0)) * right
 
 
 def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, i: torch.Tensor, f: torch.Tensor, state: dict) -> torch.Tensor:
@@ -204,11 +215,14 @@ def matrix_memory(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, i: torch.Te
 
 
 def mlstm(h: torch.Tensor, p: Mapping[str, torch.Tensor], m: Mapping[str, Any], eps: float, state: dict) -> torch.Tensor:
-    n, H, d, dv, cap = h.shape[0], m["heads"], m["dim"], m["vdim"], float(m["gate_cap"])
+    n, H, d, cap = h.shape[0], m["heads"], m["dim"], float(m.get("gate_cap") or 0.0)
+    dv = m.get("vdim") or d
     q = (h @ p["q"].t()).view(n, H, d) * d ** -0.5
     k, v = (h @ p["k"].t()).view(n, H, d), (h @ p["v"].t()).view(n, H, dv)
-    i = cap * torch.tanh((h @ p["i"].t() + p["i.b"]) / cap)
-    f = log_sigmoid(cap * torch.tanh((h @ p["f"].t() + p["f.b"]) / cap))
+    i, f = h @ p["i"].t() + p["i.b"], h @ p["f"].t() + p["f.b"]
+    if cap:                                          # (no cap: the gates' pre-activations as they are)
+        i, f = cap * torch.tanh(i / cap), cap * torch.tanh(f / cap)
+    f = log_sigmoid(f)
     o = rms(matrix_memory(q, k, v, i, f, state), eps).reshape(n, H * dv) * p["norm"]
     return (o * sigmoid(h @ p["g"].t())) @ p["o"].t()
 
@@ -295,7 +309,7 @@ def greedy_generate(cfg: Mapping[str, Any], tensors: Mapping[str, torch.Tensor],
 # ------------------------------------------------------------------------------ weights of a test model
 
 def attention_shapes(p: str, m: Mapping[str, Any], w: int, maps: int, own_kv: bool) -> dict:
-    H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+    H, G, d, dv, _ = attention_sizes(m)
     out = {p + "q": (H * maps * d, w), p + "q.b": (H * maps * d,), p + "o": (w, H * dv)}
     if own_kv:
         out.update({p + "k": (G * maps * d, w), p + "k.b": (G * maps * d,), p + "v": (G * dv, w), p + "v.b": (G * dv,)})
@@ -310,7 +324,8 @@ def tensor_shapes(cfg: Mapping[str, Any]) -> dict:
         p, m = f"l{i}.", layer["mixer"]
         out[p + "norm1"] = (w,)
         if layer["type"] == "mlstm":
-            H, d, dv = m["heads"], m["dim"], m["vdim"]
+            H, d = m["heads"], m["dim"]
+            dv = m.get("vdim") or d
             out.update({p + "mix.q": (H * d, w), p + "mix.k": (H * d, w), p + "mix.v": (H * dv, w), p + "mix.g": (H * dv, w),
                         p + "mix.o": (w, H * dv), p + "mix.norm": (H * dv,), p + "mix.i": (H, w), p + "mix.i.b": (H,),
                         p + "mix.f": (H, w), p + "mix.f.b": (H,)})
@@ -322,7 +337,8 @@ def tensor_shapes(cfg: Mapping[str, Any]) -> dict:
         else:
             out.update(attention_shapes(p + "mix.left.", m["left"], w, 1, True))
             r = m["right"]
-            H, d, dv = r["heads"], r["dim"], r["vdim"]
+            H, d = r["heads"], r["dim"]
+            dv = r.get("vdim") or d
             out.update({p + "mix.right.q": (H * d, w), p + "mix.right.k": (H * d, w), p + "mix.right.v": (H * dv, w),
                         p + "mix.right.g": (H * dv, w), p + "mix.right.o": (w, H * dv), p + "mix.right.norm": (H * dv,)})
         f = layer.get("mlp")
