@@ -293,13 +293,38 @@ def zarinex_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
             "layers": [{"type": order[i % 4], "mixer": mixers[order[i % 4]], "mlp": mlp} for i in range(layers)]}
 
 
+def betepel_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
+    """A Betepel of sizes that resemble a real model's layers, in the order differential attention, pair, matrix
+    memory, differential attention on the first one's keys and values: the differential attention with half as
+    many heads, each of two maps of 64 over values of 128, under a window of the chunk's size that keeps the
+    first 64 positions, llama3-scaled rotation of half a head; the pair's attention with heads of 64 under the
+    same window beside decayed linear attention with heads of 64; the matrix memory with heads of 64; every
+    layer with the mixture of experts that every other Miberax layer has (32 experts of an eighth of the Llama
+    layer's hidden size, four chosen, here by a table, beside a shared expert of a quarter)."""
+    rot = {"dims": 32, "base": 1e6, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    diff = {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.5,
+            "mask": {"size": chunk, "keep_first": 64}, "rot": rot}
+    pair = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": chunk},
+                     "rot": {"dims": 64, "base": 1e6}},
+            "right": {"heads": heads, "dim": 64, "vdim": 64, "decay": [1.0 - 2.0 ** -(3 + 5 * h / heads) for h in range(heads)]},
+            "left_scale": 0.8, "right_scale": 0.5}
+    memory = {"heads": heads, "dim": 64, "vdim": 64, "gate_cap": 15.0}
+    mlp = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 32, "top": 4}, "shared": {"ff": ff // 4}}
+    out = []
+    for i in range(layers):
+        kind = ("attention", "parallel", "mlstm", "attention")[i % 4]
+        mixer = dict(diff, kv_from=i - 3) if i % 4 == 3 else {"attention": diff, "parallel": pair, "mlstm": memory}[kind]
+        out.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Betepel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.25, "layers": out}
+
+
 DESIGN_SIZES = {  # width, heads (of 64), kv heads, feed-forward, layers, vocabulary, attention chunk
     "1024": (1024, 16, 4, 4096, 8, 32000, 1024),
     "2048": (2048, 32, 8, 8192, 8, 32000, 2048),
 }
 
 
-BESIDE = {"miberax": "makodra and ", "zarinex": "miberax and "}
+BESIDE = {"miberax": "makodra and ", "zarinex": "miberax and ", "betepel": "miberax and "}
 
 
 def design_compare(args):
@@ -313,10 +338,12 @@ def design_compare(args):
     for name in args.design_sizes.split(","):
         width, heads, kv_heads, ff, layers, vocab, chunk = DESIGN_SIZES[name]
         shapes = {
+            **({"betepel": betepel_shape(width, heads, kv_heads, ff, layers, vocab, chunk)} if args.design == "betepel" else {}),
             **({"zarinex": zarinex_shape(width, heads, kv_heads, ff, layers, vocab, chunk)} if args.design == "zarinex" else {}),
             **({"miberax": miberax_shape(width, heads, kv_heads, ff, layers, vocab, chunk)}
-               if args.design in ("miberax", "zarinex") else {}),
-            **({"makodra": makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk)} if args.design != "zarinex" else {}),
+               if args.design in ("miberax", "zarinex", "betepel") else {}),
+            **({"makodra": makodra_shape(width, heads, kv_heads, ff, layers, vocab, chunk)}
+               if args.design in ("makodra", "miberax") else {}),
             "llama": dict(LLAMA_3_2_1B, vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
                           num_attention_heads=heads, num_key_value_heads=kv_heads, head_dim=64),
         }
@@ -431,13 +458,13 @@ def main() -> int:
                     help="prompt length of --only-prefill (the line of the default run always has 2,048)")
     ap.add_argument("--portion", type=int, default=None,
                     help="with --only-prefill: the prompt runs in steps of at most this many tokens")
-    ap.add_argument("--design", default=None, choices=["makodra", "miberax", "zarinex"],
+    ap.add_argument("--design", default=None, choices=["makodra", "miberax", "zarinex", "betepel"],
                     help="instead of the default run: prefill (2,048 and 8,192 tokens) and decode (batch 1, 8, 64 at "
                          "--context) of this design beside the Llama decoder at equal sizes, random weights")
     ap.add_argument("--design-sizes", default="1024,2048", help="widths of --design, of " + ", ".join(DESIGN_SIZES))
     ap.add_argument("--design-phases", default="prefill2048,prefill8192,decode_b1,decode_b8,decode_b64",
                     help="with --design: which of these measurements to make")
-    ap.add_argument("--design-only", default=None, choices=["makodra", "miberax", "zarinex", "llama"],
+    ap.add_argument("--design-only", default=None, choices=["makodra", "miberax", "zarinex", "betepel", "llama"],
                     help="with --design: measure this one of the pair alone (for profiling)")
     args = ap.parse_args()
     if args.gpus != 1:

@@ -262,6 +262,29 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   }
 }
 
+// The same for one head that spans a long row: a workgroup a row.
+template <typename T, int RULE>
+__global__ __launch_bounds__(256) void row_norm_gate_kernel(const float* __restrict__ o, int64_t o_stride,
+                                                            const float* __restrict__ g_pre, int64_t g_stride,
+                                                            const float* __restrict__ norm_w, float eps, T* __restrict__ out,
+                                                            int64_t out_stride, int dim, const float* __restrict__ den) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const float* oh = o + row * o_stride;
+  const float dn = den != nullptr ? 1.f / den[row] : 1.f;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < dim; c += blockDim.x) ss += (oh[c] * dn) * (oh[c] * dn);
+  const float r = dn / sqrtf(block_sum(ss, scratch) / (float)dim + eps);
+  for (int c = threadIdx.x; c < dim; c += blockDim.x) {
+    float gate = 1.f;
+    if (RULE != GATE_NONE) {
+      const float g = g_pre[row * g_stride + c];
+      gate = RULE == RULE_DELTA ? 1.f / (1.f + expf(-g)) : g / (1.f + expf(-g));
+    }
+    out[row * out_stride + c] = from_f32<T>(oh[c] * r * norm_w[c] * gate);
+  }
+}
+
 template <int RULE>
 static int launch_scan(const ScanArgs& p, int entries, int rows, int dim, int out_is_bf16, hipStream_t stream) {
   // sixteen lanes a column (four columns a wave) where the head's size is a multiple of 16, else eight
@@ -338,7 +361,13 @@ extern "C" int dli_head_norm_gate(const float* o, int64_t o_stride, const float*
     return DLI_ERR_ARGUMENT;
   const dim3 grid(rows, (heads + 3) / 4);
   if (grid.y > 65535) return DLI_ERR_ARGUMENT;
-#define HNG(T, RULE) head_norm_gate_kernel<T, RULE><<<grid, 256, 0, stream>>>(o, o_stride, g_pre, g_stride, norm_w, eps, (T*)out, out_stride, heads, dim, den)
+#define HNG(T, RULE)                                                                                                     \
+  do {                                                                                                                   \
+    if (heads == 1 && dim > 256)                                                                                         \
+      row_norm_gate_kernel<T, RULE><<<rows, 256, 0, stream>>>(o, o_stride, g_pre, g_stride, norm_w, eps, (T*)out, out_stride, dim, den); \
+    else                                                                                                                 \
+      head_norm_gate_kernel<T, RULE><<<grid, 256, 0, stream>>>(o, o_stride, g_pre, g_stride, norm_w, eps, (T*)out, out_stride, heads, dim, den); \
+  } while (0)
   if (out_is_bf16) { if (gate == GATE_NONE) HNG(bf16_t, GATE_NONE); else if (gate) HNG(bf16_t, RULE_BONUS); else HNG(bf16_t, RULE_DELTA); }
   else { if (gate == GATE_NONE) HNG(float, GATE_NONE); else if (gate) HNG(float, RULE_BONUS); else HNG(float, RULE_DELTA); }
 #undef HNG

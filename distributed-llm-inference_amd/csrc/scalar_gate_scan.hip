@@ -22,6 +22,8 @@
 //                      A wave an (entry, head); 64 tokens at a time: with F the running sum of f inside the
 //                      block, m_t = F_t + max(m_in, max_(s <= t)(i_s - F_s)), two scans over the lanes
 //   scalar_gate_scan   the recurrence
+//   silu_columns       silu in place on some columns of a float32 matrix (a step with portions applies it to q, k and v
+//                      beforehand, all threads at once; inside the scan it would sit on the one wave that walks the tokens)
 //
 // The scan: one wave takes one (entry, head, slice of 4 columns). Sixteen lanes (a DPP row) share a column: lane
 // (col, part) keeps S[part's D/16 keys][col] in registers, and a token's sum over the keys meets in four DPP
@@ -55,17 +57,20 @@ __device__ __forceinline__ float sg_row_sum(float x) {
 
 __device__ __forceinline__ float sg_act(float x, int silu) { return silu ? x / (1.f + expf(-x)) : x; }
 
-// NK keys a lane, D = 16 NK; TB tokens staged at once (1 in a step of single tokens).
-template <int NK, int TB>
+// NK keys a lane, D = 16 NK; TB tokens staged at once (1 in a step of single tokens). GATED: keep and write factors
+// per token (else the head's constant decay and one), and with them the column of n and the denominators; SILU:
+// q, k and v pass through silu on their way into LDS. No load hangs on a condition (what is not wanted is read
+// from a clamped place and dropped), so that a batch's loads stay in flight while the chain of the one before runs.
+template <int NK, int TB, bool GATED, bool SILU>
 __global__ __launch_bounds__(64) void scalar_gate_scan_kernel(SgArgs p) {
   constexpr int D = NK * 16, COLS = 4, PER = (TB * D + 63) / 64;
   __shared__ float sk[PER * 64], sq[PER * 64], sv[TB * COLS], sa[TB], sb[TB], sfl[TB];
   const int lane = threadIdx.x, vloc = lane / 16, part = lane % 16;
   const int entry = blockIdx.x, head = blockIdx.y;
-  const int V = p.vdim, VX = V + (p.floor != nullptr ? 1 : 0);
+  const int V = p.vdim, VX = V + (GATED ? 1 : 0);
   const int my_col = (int)blockIdx.z * COLS + vloc;
   const int col = min(my_col, VX - 1);          // lanes past the last column repeat it and store nothing
-  const bool live = my_col < VX, is_n = p.floor != nullptr && col == V;
+  const bool live = my_col < VX, is_n = GATED && col == V;
   const int row0 = p.q_start[entry], n_rows = p.q_start[entry + 1] - row0;
   if (n_rows <= 0) return;
   const int64_t qk_col = (int64_t)head * D, v_col = (int64_t)head * V;
@@ -77,7 +82,7 @@ __global__ __launch_bounds__(64) void scalar_gate_scan_kernel(SgArgs p) {
     const float old = st[i];
     s[i] = fresh ? 0.f : old;
   }
-  const float decay = p.keep == nullptr ? p.decay[head] : 1.f;
+  const float decay = GATED ? 1.f : p.decay[head];
   float pk[PER], pq[PER], pv = 0.f, pa = 1.f, pb = 1.f, pf = 0.f;
   auto fetch = [&](int t0) {
 #pragma unroll
@@ -87,16 +92,16 @@ __global__ __launch_bounds__(64) void scalar_gate_scan_kernel(SgArgs p) {
       pk[m] = p.k[row * p.k_stride + qk_col + c];
       pq[m] = p.q[row * p.q_stride + qk_col + c];
     }
-    if (lane < TB * COLS) {
-      const int64_t row = row0 + min(t0 + lane / COLS, n_rows - 1);
+    {
+      const int64_t row = row0 + min(t0 + min(lane / COLS, TB - 1), n_rows - 1);
       const int c = (int)blockIdx.z * COLS + lane % COLS;
       pv = p.v[row * p.v_stride + v_col + min(c, V - 1)];
     }
-    if (lane < TB && p.keep != nullptr) {
-      const int64_t row = row0 + min(t0 + lane, n_rows - 1);
+    if (GATED) {
+      const int64_t row = row0 + min(t0 + min(lane, TB - 1), n_rows - 1);
       pa = p.keep[row * p.gate_stride + head];
       pb = p.write[row * p.gate_stride + head];
-      if (p.floor != nullptr) pf = p.floor[row * p.gate_stride + head];
+      pf = p.floor[row * p.gate_stride + head];
     }
   };
   auto step = [&](int t, int64_t row) {
@@ -119,19 +124,19 @@ __global__ __launch_bounds__(64) void scalar_gate_scan_kernel(SgArgs p) {
   for (int t0 = 0; t0 < n_rows; t0 += TB) {
 #pragma unroll
     for (int m = 0; m < PER; ++m) {
-      sk[lane + 64 * m] = sg_act(pk[m], p.silu);
-      sq[lane + 64 * m] = sg_act(pq[m], p.silu) * p.q_scale;
+      sk[lane + 64 * m] = sg_act(pk[m], SILU);
+      sq[lane + 64 * m] = sg_act(pq[m], SILU) * p.q_scale;
     }
     if (lane < TB * COLS) {
       const int c = (int)blockIdx.z * COLS + lane % COLS;
-      sv[lane] = p.floor != nullptr && c >= V ? 1.f : sg_act(pv, p.silu);   // the column of n reads a value of one
+      sv[lane] = GATED && c >= V ? 1.f : sg_act(pv, SILU);   // the column of n reads a value of one
     }
     if (lane < TB) {
-      sa[lane] = p.keep != nullptr ? pa : decay;
+      sa[lane] = GATED ? pa : decay;
       sb[lane] = pb;
       sfl[lane] = pf;
     }
-    if (TB > 1 && t0 + TB < n_rows) fetch(t0 + TB);  // on their way while the chain below runs
+    if (TB > 1) fetch(t0 + TB);  // on their way while the chain below runs (past the last row: the last row again, dropped)
     __syncthreads();
     const int nb = min(TB, n_rows - t0);
     if (nb == TB) {
@@ -237,7 +242,25 @@ __global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__
   if (lane == 0) *ms = m_in;
 }
 
+// x [rows][stride] float32: the first `width` columns become silu of themselves. A thread an element.
+__global__ void silu_columns_kernel(float* __restrict__ x, int64_t stride, int width) {
+  const int64_t row = blockIdx.x;
+  const int i = blockIdx.y * blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  const float v = x[row * stride + i];
+  x[row * stride + i] = v / (1.f + expf(-v));
+}
+
 extern "C" {
+
+int dli_silu_columns(float* x, int64_t stride, int rows, int width, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0 || stride < width) return DLI_ERR_ARGUMENT;
+  const dim3 grid(rows, (width + 255) / 256);
+  if (grid.y > 65535) return DLI_ERR_ARGUMENT;
+  silu_columns_kernel<<<grid, 256, 0, stream>>>(x, stride, width);
+  return dli_launch_status();
+}
 
 int dli_exp_gates(const float* pre, int64_t stride, int i_off, int f_off, const float* i_bias, const float* f_bias, float cap,
                   float* state, int64_t state_stride, int64_t m_off, const int* q_start, const int* positions,
@@ -276,12 +299,19 @@ int dli_scalar_gate_scan(const float* q, int64_t q_stride, const float* k, int64
   const bool single = rows == entries;
   const dim3 grid(entries, heads, (vx + 3) / 4);
   if (grid.z > 65535) return DLI_ERR_ARGUMENT;
+  const bool gated = keep != nullptr;
+  if (gated && floor == nullptr) return DLI_ERR_ARGUMENT;   // (gates without a normaliser: no model asks for them yet)
+#define SG_LAUNCH(NK, TBV)                                                                                  \
+  {                                                                                                         \
+    if (gated) scalar_gate_scan_kernel<NK, TBV, true, false><<<grid, 64, 0, stream>>>(p);                  \
+    else if (silu) scalar_gate_scan_kernel<NK, TBV, false, true><<<grid, 64, 0, stream>>>(p);              \
+    else scalar_gate_scan_kernel<NK, TBV, false, false><<<grid, 64, 0, stream>>>(p);                       \
+  }
 #define SG_CASE(NK, TBM)                                                                     \
   case NK * 16:                                                                              \
-    if (single) scalar_gate_scan_kernel<NK, 1><<<grid, 64, 0, stream>>>(p);                  \
-    else scalar_gate_scan_kernel<NK, TBM><<<grid, 64, 0, stream>>>(p);                       \
+    if (single) SG_LAUNCH(NK, 1) else SG_LAUNCH(NK, TBM)                                     \
     break;
-  switch (dim) {
+  switch (gated && silu ? -1 : dim) {   // (silu under gates: the slow kernel takes every combination)
     SG_CASE(1, 16) SG_CASE(2, 16) SG_CASE(3, 16) SG_CASE(4, 16) SG_CASE(5, 8) SG_CASE(6, 8) SG_CASE(7, 8) SG_CASE(8, 8)
     SG_CASE(12, 4) SG_CASE(16, 4)
     default: {
@@ -291,6 +321,7 @@ int dli_scalar_gate_scan(const float* q, int64_t q_stride, const float* k, int64
     }
   }
 #undef SG_CASE
+#undef SG_LAUNCH
   return dli_launch_status();
 }
 

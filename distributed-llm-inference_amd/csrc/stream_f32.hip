@@ -26,6 +26,8 @@
 //   diff_head_norm     two attention maps over the same values combined head by head: a1 - lambda a2, divided by
 //                      its root mean square over the head, times a constant and a sigmoid gate per head
 //   scale_f32          y *= c in place
+//   rms_norm_pair      two norms of the same row (two weights) from one pass over its statistics
+//   add_pair_into_stream  x += a + b
 #include "common.h"
 
 template <typename T>
@@ -407,6 +409,31 @@ __global__ void scale_f32_kernel(float* __restrict__ y, int64_t n, float scale) 
   if (i < n) y[i] *= scale;
 }
 
+// Two norms of the same float32 row with one pass over its statistics: out1 = w1 * x * r, out2 = w2 * x * r,
+// r = 1 / sqrt(mean(x^2) + eps) (a mixer and a feed-forward that read the same stream behind norms of their own).
+template <typename T>
+__global__ void rms_norm_pair_kernel(const float* __restrict__ x, const float* __restrict__ w1, const float* __restrict__ w2,
+                                     T* __restrict__ out1, T* __restrict__ out2, int width, float eps) {
+  __shared__ float scratch[16];
+  const int64_t row = blockIdx.x;
+  const float* xr = x + row * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) ss += xr[i] * xr[i];
+  const float r = 1.f / sqrtf(block_sum(ss, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    const float v = xr[i] * r;
+    out1[row * width + i] = from_f32<T>(w1[i] * v);
+    out2[row * width + i] = from_f32<T>(w2[i] * v);
+  }
+}
+
+// x += a + b: two sublayers' results are added to each other and then into the stream. A thread an element.
+__global__ void add_pair_into_stream_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
+                                            int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) x[i] += a[i] + b[i];
+}
+
 extern "C" {
 
 int dli_embed_sinusoid(const void* table, const int* ids, const int* positions, const float* inv_freq, float* out,
@@ -623,6 +650,26 @@ int dli_scale_f32(float* y, int64_t n, float scale, hipStream_t stream) {
   const int64_t blocks = (n + 255) / 256;
   if (blocks > 0x7fffffff) return DLI_ERR_ARGUMENT;
   scale_f32_kernel<<<(unsigned)blocks, 256, 0, stream>>>(y, n, scale);
+  return dli_launch_status();
+}
+
+int dli_rms_norm_pair(const float* x, const float* w1, const float* w2, void* out1, void* out2, int rows, int width, float eps,
+                      int is_bf16, hipStream_t stream) {
+  if (rows <= 0) return DLI_OK;
+  if (width <= 0) return DLI_ERR_ARGUMENT;
+  const int threads = width >= 2048 ? 512 : 256;
+  if (is_bf16)
+    rms_norm_pair_kernel<bf16_t><<<rows, threads, 0, stream>>>(x, w1, w2, (bf16_t*)out1, (bf16_t*)out2, width, eps);
+  else
+    rms_norm_pair_kernel<float><<<rows, threads, 0, stream>>>(x, w1, w2, (float*)out1, (float*)out2, width, eps);
+  return dli_launch_status();
+}
+
+int dli_add_pair_into_stream(float* x, const float* a, const float* b, int64_t n, hipStream_t stream) {
+  if (n <= 0) return DLI_OK;
+  const int64_t blocks = (n + 255) / 256;
+  if (blocks > 0x7fffffff) return DLI_ERR_ARGUMENT;
+  add_pair_into_stream_kernel<<<(unsigned)blocks, 256, 0, stream>>>(x, a, b, n);
   return dli_launch_status();
 }
 

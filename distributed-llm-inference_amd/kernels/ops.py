@@ -144,6 +144,9 @@ _SIGNATURES = {
                            _c_int, _c_int, _c_ptr],
     "dli_branch_weighted_sum": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_ptr],
     "dli_scale_f32": [_c_ptr, _c_i64, _c_float, _c_ptr],
+    "dli_silu_columns": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr],
+    "dli_rms_norm_pair": [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_float, _c_int, _c_ptr],
+    "dli_add_pair_into_stream": [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "dli_table_choose": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "dli_exp_gates": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr,
                       _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
@@ -2334,3 +2337,31 @@ def table_choose(table: torch.Tensor, token_ids: torch.Tensor, ids: torch.Tensor
     _require(table.shape[1] == top and token_ids.shape[0] == n and weights.shape == (n, top), "table, ids and weights disagree")
     _check(library().dli_table_choose(_ptr(table), _ptr(token_ids), n, top, table.shape[0], _ptr(ids), _ptr(weights), _stream()),
            "table_choose")
+
+
+def rms_norm_pair(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, eps: float, out1: torch.Tensor, out2: torch.Tensor) -> None:
+    """``out1 = w1 * x / sqrt(mean(x^2) + eps)`` and ``out2`` alike with ``w2``: two norms of one float32 ``x`` that
+    agree on eps, from one pass over the rows' statistics; both rounded once to the outputs' type."""
+    _dense(x, "x", torch.float32, 2)
+    for name, w in (("w1", w1), ("w2", w2)):
+        _dense(w, name, torch.float32, 1)
+        _require(w.shape[0] == x.shape[1], f"{name} must hold a value per column")
+    _dense(out1, "out1", ndim=2)
+    _dense(out2, "out2", out1.dtype, 2)
+    _require(out1.shape == x.shape and out2.shape == x.shape, "the outputs differ from x in shape")
+    _check(library().dli_rms_norm_pair(_ptr(x), _ptr(w1), _ptr(w2), _ptr(out1), _ptr(out2), x.shape[0], x.shape[1], float(eps),
+                                       _is_bf16(out1.dtype), _stream()), "rms_norm_pair")
+
+
+def add_pair_into_stream(x: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> None:
+    """``x += a + b`` (all float32, equal shapes): the two results are added to each other first."""
+    for name, t in (("x", x), ("a", a), ("b", b)):
+        _dense(t, name, torch.float32, 2)
+    _require(a.shape == x.shape and b.shape == x.shape, "a and b differ from x in shape")
+    _check(library().dli_add_pair_into_stream(_ptr(x), _ptr(a), _ptr(b), x.numel(), _stream()), "add_pair_into_stream")
+
+
+def silu_columns(x: torch.Tensor) -> None:
+    """``x <- silu(x)`` in place: float32 ``[n, width]`` with contiguous rows (columns of a wider matrix will do)."""
+    _f32_rows(x, "x")
+    _check(library().dli_silu_columns(_ptr(x), x.stride(0), x.shape[0], x.shape[1], _stream()), "silu_columns")

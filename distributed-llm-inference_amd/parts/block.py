@@ -197,11 +197,20 @@ class ParallelNormsBlock(Block):
             raise RuntimeError("the parallel_norms block keeps a float32 residual stream")
         if delta is not None:
             ops.add(x, delta, x)
-        y = _as_f32(parts["mixer"].forward(parts["mixer_norm"].forward(x), ctx, cache))
-        if "feed_forward" in parts:
-            f = _as_f32(parts["feed_forward"].forward(parts["feed_forward_norm"].forward(x), ctx))
-            ops.add(y, f, y)
-        ops.add(x, y, x)
+        if "feed_forward" not in parts:
+            ops.add(x, _as_f32(parts["mixer"].forward(parts["mixer_norm"].forward(x), ctx, cache)), x)
+            return x, None
+        n1, n2 = parts["mixer_norm"], parts["feed_forward_norm"]
+        pair = [getattr(n, "fused_params", None) for n in (n1, n2)]
+        if all(pair) and pair[0]()[1] == pair[1]()[1]:
+            # plain RMS norms that agree on eps: one pass over the rows' statistics for both
+            h1, h2 = self.rt.empty(*x.shape), self.rt.empty(*x.shape)
+            ops.rms_norm_pair(x, pair[0]()[0], pair[1]()[0], pair[0]()[1], h1, h2)
+        else:
+            h1, h2 = n1.forward(x), n2.forward(x)
+        y = _as_f32(parts["mixer"].forward(h1, ctx, cache))
+        f = _as_f32(parts["feed_forward"].forward(h2, ctx))
+        ops.add_pair_into_stream(x, y, f)
         return x, None
 
 

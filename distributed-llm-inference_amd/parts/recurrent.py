@@ -429,8 +429,13 @@ class DecayedLinear(_ScalarGateMixer):
             self.finalize()
         k0, v0, g0 = self.hd, 2 * self.hd, 2 * self.hd + self.hv
         o = torch.empty(n, self.hv, device=self.rt.device, dtype=torch.float32)
+        # a step of single tokens applies silu inside the scan; one with portions beforehand, all threads at once
+        # (inside, it would sit on the one wave that walks a request's tokens)
+        inside = ctx.num_decode == ctx.num_entries
+        if not inside:
+            ops.silu_columns(proj[:, :g0])
         ops.scalar_gate_scan(proj[:, :k0], proj[:, k0:v0], proj[:, v0:g0], state, ctx.q_start, ctx.positions, ctx.state_slots,
-                             o, self.num_heads, self.head_dim, self.value_dim, decay=self.decay, silu=True)
+                             o, self.num_heads, self.head_dim, self.value_dim, decay=self.decay, silu=inside)
         out = self.rt.empty(n, self.hv)
         # one norm over all heads: the row as a single head
         ops.head_norm_gate(o, proj[:, g0:g0 + self.hv], self.norm_w, self.norm_eps, out, 1, self.hv, gate="sigmoid")
