@@ -30,12 +30,20 @@ def build_betepel_spec(cfg: BetepelConfig) -> ModelSpec:
                                        low_freq_factor=r.low, high_freq_factor=r.high,
                                        original_max_position_embeddings=r.original))
 
-    def attention(a: BetepelAttention, prefix: str) -> PartSpec:
+    def kept_keys(i: int) -> Optional[int]:
+        """What layer ``i``'s pages must keep for itself and for the layers that read them: every key (0) if one of
+        them sees every earlier position or keeps first positions, else the longest of their windows."""
+        readers = [cfg.layers[i].attention] + [l.attention for l in cfg.layers if l.type == "attention" and l.attention.kv_from == i]
+        if len(readers) == 1:
+            return None
+        return 0 if any(not a.window or a.keep_first for a in readers) else max(a.window for a in readers)
+
+    def attention(a: BetepelAttention, prefix: str, cache_window: Optional[int] = None) -> PartSpec:
         params = dict(hidden_size=w, num_heads=a.heads, num_kv_heads=a.kv_heads, head_dim=a.dim, value_dim=a.vdim,
                       scale=a.scale, qk_unit=False, position=position(a), window=a.window, keep_first=a.keep_first,
                       bias=True, norm_eps=eps)
         if a.diff is not None:
-            params.update(maps=2, diff=a.diff, head_gate=True, own_kv=a.kv_from is None)
+            params.update(maps=2, diff=a.diff, head_gate=True, own_kv=a.kv_from is None, cache_window=cache_window)
         return PartSpec("scored_attention", params, prefix)
 
     def memory(m: BetepelMemory, prefix: str) -> PartSpec:
@@ -51,7 +59,7 @@ def build_betepel_spec(cfg: BetepelConfig) -> ModelSpec:
         if layer.type == "mlstm":
             mixer = memory(layer.memory, p + "mix.")
         elif layer.type == "attention":
-            mixer = attention(layer.attention, p + "mix.")
+            mixer = attention(layer.attention, p + "mix.", kept_keys(i) if layer.attention.kv_from is None else None)
         else:
             mixer = PartSpec("parallel_mixers", dict(
                 hidden_size=w, combine="weighted_sum", scales={"left": layer.left_scale, "right": layer.right_scale},

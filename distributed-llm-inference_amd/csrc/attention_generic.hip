@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       const int j = j0 + r;
       float kv = 0.f;
       if (j < j_end) {
-        const int64_t page = table[j / page_size];
+        const int64_t page = max(table[j / page_size], 0);   // (a page that a window has passed: any page, its keys are not seen)
         kv = to_f32(k_pages[((page * kv_heads + kvh) * page_size + j % page_size) * head_dim + c]);
       }
       ks[r][c] = kv;
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(256) void attention_generic_kernel(
       const int j = j0 + r;
       float vv = 0.f;
       if (j < j_end) {
-        const int64_t page = table[j / page_size];
+        const int64_t page = max(table[j / page_size], 0);   // (a page that a window has passed: any page, its keys are not seen)
         vv = to_f32(v_pages[((page * sc.v_heads + vh) * value_dim + c) * page_size + j % page_size]);
       }
       vs[r][c] = vv;
@@ -293,7 +293,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
     const bool seen = j <= pos && j >= j_lo && (j >= j_begin || j < keep);
     // the page of this lane's key, for its own row of K and, handed round, for the rows of V (a key
     // past the request's last page reads the table's last entry: its weight is zero)
-    const int my_page = table[min(j / page_size, table_stride - 1)];
+    const int my_page = max(table[min(j / page_size, table_stride - 1)], 0);
     float s[GQ];
 #pragma unroll
     for (int h = 0; h < GQ; ++h) s[h] = 0.f;
@@ -372,7 +372,7 @@ __global__ __launch_bounds__(512) void attention_scored_decode_kernel(
         int jj = first;
         while (jj <= last) {
           const int jk = j0 + jj;
-          const int64_t page = table[jk / page_size];
+          const int64_t page = max(table[jk / page_size], 0);
           const int off = jk % page_size;
           const T* vr = v_pages + ((page * sc.v_heads + vh) * value_dim + col) * page_size + off;
           if (v_packs && off % PN == 0 && jj + PN - 1 <= last) {

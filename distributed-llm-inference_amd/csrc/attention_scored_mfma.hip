@@ -83,7 +83,7 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
 #pragma unroll
     for (int sub = 0; sub < 4; ++sub) {
       const int key = j0 + 16 * sub + col;              // the key whose row this lane reads
-      const int64_t page = table[min(key / ps, a.table_stride - 1)];
+      const int64_t page = max(table[min(key / ps, a.table_stride - 1)], 0);   // (a page that a window has passed: any page will do)
       const bf16_t* kr = a.k_pages + ((page * G + kvh) * ps + key % ps) * D + 4 * grp;
       float4s c = float4s{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(256) void attention_scored_mfma_kernel(ScoredArgs a
 #pragma unroll
     for (int sub = 0; sub < 4; ++sub) {
       const int key = j0 + 16 * sub + 4 * grp;          // the four keys whose values this lane reads, one value row a product
-      const int64_t page = table[min(key / ps, a.table_stride - 1)];
+      const int64_t page = max(table[min(key / ps, a.table_stride - 1)], 0);   // (a page that a window has passed: any page will do)
       const bf16_t* vr = a.v_pages + ((page * GV + vh) * V + col) * ps + key % ps;
 #pragma unroll
       for (int t = 0; t < VT; ++t)

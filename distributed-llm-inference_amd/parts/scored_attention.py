@@ -86,8 +86,13 @@ class ScoredAttention(Mixer):
                  sink: bool = False, output_gate: bool = False, value_mix: str = "none",
                  value_mix_key: str = "first_values", names: Optional[Mapping[str, str]] = None,
                  position: Optional[PartSpec] = None, bias: bool = False, keep_first: int = 0, maps: int = 1,
-                 diff: float = 0.0, head_gate: bool = False, own_kv: bool = True) -> None:
+                 diff: float = 0.0, head_gate: bool = False, own_kv: bool = True, cache_window: Optional[int] = None) -> None:
+        """``cache_window``: how many of the latest keys the pages must keep where that is not this layer's own
+        window (0: all): other layers that read this layer's cache may look further back than it does."""
         super().__init__(runtime)
+        if cache_window is not None and (cache_window < 0 or (cache_window and (not window or keep_first or cache_window < window))):
+            raise ValueError("scored_attention: the pages must keep at least what this layer's own mask sees")
+        self.cache_window = cache_window
         if maps not in (1, 2):
             raise ValueError("one score map a head, or two whose results are subtracted")
         if maps == 2 and (qk_unit or output_gate or value_mix != "none"):
@@ -207,7 +212,8 @@ class ScoredAttention(Mixer):
         if not self.own_kv:
             return None   # the schedule hands this layer another entry's cache
         # (a window that keeps its first positions gives no page back while the request runs)
-        return PagedKVSpec(self.num_kv_heads * self.maps, self.head_dim, 0 if self.keep_first else self.window,
+        kept = self.cache_window if self.cache_window is not None else (0 if self.keep_first else self.window)
+        return PagedKVSpec(self.num_kv_heads * self.maps, self.head_dim, kept,
                            None if self.value_dim == self.head_dim else self.value_dim,
                            self.num_kv_heads if self.maps > 1 else None)
 
