@@ -189,6 +189,198 @@ __global__ void scalar_gate_any_kernel(SgArgs p, int D) {
   }
 }
 
+// Steps with portions, heads of 16 to 64 keys in steps of 16: the same recurrence 64 tokens at a time on the matrix
+// cores, all in 32-bit (v_mfma_f32_16x16x4_f32). With A_t the running sum of log a inside the chunk (never above zero,
+// so every factor below is at most one), w_s = exp(A_last - A_s) b_s and S the state before the chunk:
+//
+//   P[t][s] = (q_t . k_s) exp(A_t - A_s) b_s  for s <= t,   o_t = sum_s P[t][s] v_s + exp(A_t) S^T q_t,
+//   S <- exp(A_last) S + sum_s w_s k_s v_s^T,
+//
+// and for the matrix memory n_t . q_t = sum_s P[t][s] + exp(A_t) (n . q_t), n <- exp(A_last) n + sum_s w_s k_s.
+// A workgroup of four waves takes one (entry, head, slice of 16 value columns) and walks the entry's chunks in
+// order, the next chunk's rows on their way into registers while this one is multiplied. Q, K and P lie in LDS row by
+// row, V and the state's slice column by column (as the state is kept), every row padded by four floats: a lane
+// then reads the four k of four consecutive matrix instructions as one 16-byte access (the instructions' k may be
+// dealt to the lanes in any order as long as both operands agree: lane group g takes k = 16 step + 4 g .. + 3),
+// and sixteen rows fall into all 64 banks. Wave w makes the rows 16 w .. 16 w + 15 of P and of the chunk's
+// results, and sixteen keys' rows of the new state. Rows past the entry's last count as a = 1, b = 0 and
+// q = k = v = 0. The slice that holds column 0 also carries n and writes the denominators.
+typedef float sg_f4 __attribute__((ext_vector_type(4)));
+
+template <int D, bool GATED>
+__global__ __launch_bounds__(256) void scalar_gate_chunk_kernel(SgArgs p, const float* __restrict__ log_keep) {
+  constexpr int C = 64, VS = 16, DS = D + 4, PS = C + 4, QK_PER = C * D / 256, V_PER = C * VS / 256;
+  __shared__ __attribute__((aligned(16))) float sQ[C * DS], sK[C * DS], sP[C * PS], sVt[VS * PS], sSt[VS * DS], sW[C];
+  __shared__ float sN[D], sB[C], sFl[C];
+  __shared__ double sA[C];   // the running sums of log a: their differences are taken before rounding (a chunk's sum may
+                             // reach the hundreds, where a float's last bit is 1e-5 of the factor it stands for)
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int li = lane % 16, lk = lane / 16;                 // a matrix operand's row (or column) and its group of k; a result's column and group of four rows
+  const int entry = blockIdx.x, head = blockIdx.y, v0 = (int)blockIdx.z * VS;
+  const int V = p.vdim, VX = V + (GATED ? 1 : 0);
+  const int row0 = p.q_start[entry], n_rows = p.q_start[entry + 1] - row0;
+  if (n_rows <= 0) return;
+  const bool fresh = p.positions[row0] == 0, with_n = GATED && blockIdx.z == 0;
+  float* st = p.state + (int64_t)p.state_slots[entry] * p.state_stride + (int64_t)head * VX * D;
+  const int64_t qk_col = (int64_t)head * D, v_col = (int64_t)head * V;
+  for (int idx = tid; idx < D * VS; idx += 256) {
+    const int j = idx / D, d = idx - j * D;                 // the state keeps a column's keys side by side
+    const float old = v0 + j < V ? st[(int64_t)(v0 + j) * D + d] : 0.f;
+    sSt[j * DS + d] = fresh ? 0.f : old;
+  }
+  if (tid < D) {
+    const float old = with_n ? st[(int64_t)V * D + tid] : 0.f;
+    sN[tid] = fresh ? 0.f : old;
+  }
+  const float log_decay = GATED ? 0.f : fmaxf(logf(p.decay[head]), -1e30f);
+  float rq[QK_PER], rk[QK_PER], rv[V_PER], rla = 0.f, rb = 0.f, rfl = 0.f;
+  auto fetch = [&](int t0) {                                // rows past the last: the last row again, dropped when staged
+#pragma unroll
+    for (int m = 0; m < QK_PER; ++m) {
+      const int idx = tid + 256 * m, t = idx / D, d = idx - t * D;
+      const int64_t row = row0 + min(t0 + t, n_rows - 1);
+      rk[m] = p.k[row * p.k_stride + qk_col + d];
+      rq[m] = p.q[row * p.q_stride + qk_col + d];
+    }
+#pragma unroll
+    for (int m = 0; m < V_PER; ++m) {
+      const int idx = tid + 256 * m, t = idx / VS, j = idx - t * VS;
+      const int64_t row = row0 + min(t0 + t, n_rows - 1);
+      rv[m] = p.v[row * p.v_stride + v_col + min(v0 + j, V - 1)];
+    }
+    if (GATED) {
+      const int64_t at = (int64_t)(row0 + min(t0 + lane, n_rows - 1)) * p.gate_stride + head;
+      rla = log_keep[at];
+      rb = p.write[at];
+      rfl = p.floor[at];
+    }
+  };
+  fetch(0);
+  for (int t0 = 0; t0 < n_rows; t0 += C) {
+    const int nb = min(C, n_rows - t0);
+    __syncthreads();                                        // the chunk before has been read, the state's slice is whole
+#pragma unroll
+    for (int m = 0; m < QK_PER; ++m) {
+      const int idx = tid + 256 * m, t = idx / D, d = idx - t * D;
+      sK[t * DS + d] = t < nb ? rk[m] : 0.f;
+      sQ[t * DS + d] = t < nb ? rq[m] * p.q_scale : 0.f;
+    }
+#pragma unroll
+    for (int m = 0; m < V_PER; ++m) {
+      const int idx = tid + 256 * m, t = idx / VS, j = idx - t * VS;
+      sVt[j * PS + t] = t < nb && v0 + j < V ? rv[m] : 0.f;
+    }
+    if (wave == 0) {
+      double la = GATED ? rla : log_decay;
+      float b = GATED ? rb : 1.f;
+      if (lane >= nb) { la = 0.0; b = 0.f; }
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const double up = __shfl_up(la, d, DLI_WAVE);
+        if (lane >= d) la += up;
+      }
+      const double last = __shfl(la, 63, DLI_WAVE);
+      sA[lane] = la;
+      sB[lane] = b;
+      sW[lane] = expf((float)(last - la)) * b;
+      sFl[lane] = rfl;
+    }
+    fetch(t0 + C);                                          // the next chunk's rows, on their way while this one is multiplied
+    __syncthreads();
+    const float a_last = (float)sA[C - 1];
+    // P: this wave's sixteen rows against the key blocks up to its own
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) {
+      if (cb > wave) break;
+      sg_f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < D / 16; ++g) {
+        const sg_f4 a4 = *reinterpret_cast<const sg_f4*>(sQ + (16 * wave + li) * DS + 16 * g + 4 * lk);
+        const sg_f4 b4 = *reinterpret_cast<const sg_f4*>(sK + (16 * cb + li) * DS + 16 * g + 4 * lk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], b4[j], acc, 0, 0, 0);
+      }
+      const int s_ = 16 * cb + li;
+      const double as = sA[s_];
+      const float bs = sB[s_];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = 16 * wave + 4 * lk + r;
+        sP[t * PS + s_] = s_ <= t ? acc[r] * expf((float)(sA[t] - as)) * bs : 0.f;
+      }
+    }
+    __syncthreads();
+    {
+      sg_f4 acc = {0.f, 0.f, 0.f, 0.f}, far = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (g > wave) break;
+        const sg_f4 a4 = *reinterpret_cast<const sg_f4*>(sP + (16 * wave + li) * PS + 16 * g + 4 * lk);
+        const sg_f4 b4 = *reinterpret_cast<const sg_f4*>(sVt + li * PS + 16 * g + 4 * lk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], b4[j], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int g = 0; g < D / 16; ++g) {
+        const sg_f4 a4 = *reinterpret_cast<const sg_f4*>(sQ + (16 * wave + li) * DS + 16 * g + 4 * lk);
+        const sg_f4 b4 = *reinterpret_cast<const sg_f4*>(sSt + li * DS + 16 * g + 4 * lk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) far = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j], b4[j], far, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int t = 16 * wave + 4 * lk + r;
+        if (t < nb && v0 + li < V)
+          p.o[(int64_t)(row0 + t0 + t) * p.o_stride + v_col + v0 + li] = fmaf(expf((float)sA[t]), far[r], acc[r]);
+      }
+      if (with_n) {                                         // row t = 16 wave + li, a quarter of its sums a lane
+        const int t = 16 * wave + li;
+        float sum = 0.f, qn = 0.f;
+        for (int s_ = 16 * lk; s_ < 16 * lk + 16; ++s_) sum += s_ <= t ? sP[t * PS + s_] : 0.f;
+        for (int d = lk * (D / 4); d < (lk + 1) * (D / 4); ++d) qn = fmaf(sQ[t * DS + d], sN[d], qn);
+        sum += __shfl_xor(sum, 16, DLI_WAVE);
+        sum += __shfl_xor(sum, 32, DLI_WAVE);
+        qn += __shfl_xor(qn, 16, DLI_WAVE);
+        qn += __shfl_xor(qn, 32, DLI_WAVE);
+        if (lk == 0 && t < nb)
+          p.den[(int64_t)(row0 + t0 + t) * p.heads + head] = fmaxf(fabsf(fmaf(expf((float)sA[t]), qn, sum)), sFl[t]) + 1e-6f;
+      }
+    }
+    __syncthreads();                                        // the old state has been read by all
+    if (wave < D / 16) {
+      // the new state's keys 16 wave .. + 15 for the slice's sixteen columns: (w V)^T K, a result's row a column of the slice
+      sg_f4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const sg_f4 v4 = *reinterpret_cast<const sg_f4*>(sVt + li * PS + 16 * g + 4 * lk);
+        const sg_f4 w4 = *reinterpret_cast<const sg_f4*>(sW + 16 * g + 4 * lk);
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(v4[j] * w4[j], sK[(16 * g + 4 * lk + j) * DS + 16 * wave + li], acc, 0, 0, 0);
+      }
+      const float keep_all = expf(a_last);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float* at = sSt + (4 * lk + r) * DS + 16 * wave + li;
+        *at = fmaf(keep_all, *at, acc[r]);
+      }
+    }
+    if (with_n && tid >= 192 && tid - 192 < D) {            // (the last wave has no rows of the state to make for heads under 64)
+      const int d = tid - 192;
+      float sum = 0.f;
+#pragma unroll 8
+      for (int s_ = 0; s_ < C; ++s_) sum = fmaf(sW[s_], sK[s_ * DS + d], sum);
+      sN[d] = fmaf(expf(a_last), sN[d], sum);
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < D * VS; idx += 256) {
+    const int j = idx / D, d = idx - j * D;
+    if (v0 + j < V) st[(int64_t)(v0 + j) * D + d] = sSt[j * DS + d];
+  }
+  if (with_n && tid < D) st[(int64_t)V * D + tid] = sN[tid];
+}
+
 // pre [rows][stride]: the input gate's pre-activation of head h at column i_off + h, the forget gate's at
 // f_off + h; m of head h at state[slot][m_off + h]. keep, write, floor: [rows][heads].
 __global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__ pre, int64_t stride, int i_off, int f_off,
@@ -197,7 +389,7 @@ __global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__
                                                        int64_t m_off, const int* __restrict__ q_start,
                                                        const int* __restrict__ positions, const int* __restrict__ state_slots,
                                                        float* __restrict__ keep, float* __restrict__ write,
-                                                       float* __restrict__ floor, int heads) {
+                                                       float* __restrict__ floor, float* __restrict__ log_keep, int heads) {
   const int lane = threadIdx.x, entry = blockIdx.x, head = blockIdx.y;
   const int row0 = q_start[entry], n_rows = q_start[entry + 1] - row0;
   if (n_rows <= 0) return;
@@ -234,6 +426,7 @@ __global__ __launch_bounds__(64) void exp_gates_kernel(const float* __restrict__
     if (have) {
       const int64_t at = (row0 + t0 + lane) * (int64_t)heads + head;
       keep[at] = expf(gf + m_prev - m);
+      log_keep[at] = fminf(gf + m_prev - m, 0.f);
       write[at] = expf(gi - m);
       floor[at] = expf(-m);
     }
@@ -264,25 +457,25 @@ int dli_silu_columns(float* x, int64_t stride, int rows, int width, hipStream_t 
 
 int dli_exp_gates(const float* pre, int64_t stride, int i_off, int f_off, const float* i_bias, const float* f_bias, float cap,
                   float* state, int64_t state_stride, int64_t m_off, const int* q_start, const int* positions,
-                  const int* state_slots, float* keep, float* write, float* floor, int entries, int rows, int heads,
-                  hipStream_t stream) {
+                  const int* state_slots, float* keep, float* write, float* floor, float* log_keep, int entries, int rows,
+                  int heads, hipStream_t stream) {
   if (rows <= 0 || entries <= 0) return DLI_OK;
   if (rows < entries || heads <= 0 || heads > 65535 || i_off < 0 || f_off < 0 || i_off + heads > stride ||
       f_off + heads > stride || m_off < 0 || m_off + heads > state_stride || cap < 0.f)
     return DLI_ERR_ARGUMENT;
   exp_gates_kernel<<<dim3(entries, heads), 64, 0, stream>>>(pre, stride, i_off, f_off, i_bias, f_bias, cap, state,
                                                             state_stride, m_off, q_start, positions, state_slots, keep, write,
-                                                            floor, heads);
+                                                            floor, log_keep, heads);
   return dli_launch_status();
 }
 
 // keep, write: [rows][heads] or both nullptr (then decay [heads] and a write factor of one); floor and den
 // [rows][heads] come together, and with them the state has a column more a head.
 int dli_scalar_gate_scan(const float* q, int64_t q_stride, const float* k, int64_t k_stride, const float* v, int64_t v_stride,
-                         const float* keep, const float* write, int64_t gate_stride, const float* decay, const float* floor,
-                         float* den, float* state, int64_t state_stride, const int* q_start, const int* positions,
+                         const float* keep, const float* write, const float* log_keep, int64_t gate_stride, const float* decay,
+                         const float* floor, float* den, float* state, int64_t state_stride, const int* q_start, const int* positions,
                          const int* state_slots, float* o, int64_t o_stride, int entries, int rows, int heads, int dim,
-                         int vdim, float q_scale, int silu, hipStream_t stream) {
+                         int vdim, float q_scale, int silu, int chunked, hipStream_t stream) {
   if (rows <= 0 || entries <= 0) return DLI_OK;
   const int vx = vdim + (floor != nullptr ? 1 : 0);
   if (rows < entries || heads <= 0 || heads > 65535 || dim <= 0 || dim > 4096 || vdim <= 0 ||
@@ -301,6 +494,19 @@ int dli_scalar_gate_scan(const float* q, int64_t q_stride, const float* k, int64
   if (grid.z > 65535) return DLI_ERR_ARGUMENT;
   const bool gated = keep != nullptr;
   if (gated && floor == nullptr) return DLI_ERR_ARGUMENT;   // (gates without a normaliser: no model asks for them yet)
+  if (!single && !silu && dim % 16 == 0 && dim <= 64 && (!gated || log_keep != nullptr) && chunked) {
+    // a step with portions: chunks of 64 tokens on the matrix cores
+    const dim3 cgrid(entries, heads, (vdim + 15) / 16);
+    if (cgrid.z > 65535) return DLI_ERR_ARGUMENT;
+#define SG_CHUNK(DIM)                                                                                   \
+  case DIM:                                                                                             \
+    if (gated) scalar_gate_chunk_kernel<DIM, true><<<cgrid, 256, 0, stream>>>(p, log_keep);             \
+    else scalar_gate_chunk_kernel<DIM, false><<<cgrid, 256, 0, stream>>>(p, log_keep);                  \
+    break;
+    switch (dim) { SG_CHUNK(16) SG_CHUNK(32) SG_CHUNK(48) SG_CHUNK(64) }
+#undef SG_CHUNK
+    return dli_launch_status();
+  }
 #define SG_LAUNCH(NK, TBV)                                                                                  \
   {                                                                                                         \
     if (gated) scalar_gate_scan_kernel<NK, TBV, true, false><<<grid, 64, 0, stream>>>(p);                  \

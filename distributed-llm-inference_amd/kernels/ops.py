@@ -149,10 +149,10 @@ _SIGNATURES = {
     "dli_add_pair_into_stream": [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr],
     "dli_table_choose": [_c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr],
     "dli_exp_gates": [_c_ptr, _c_i64, _c_int, _c_int, _c_ptr, _c_ptr, _c_float, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_ptr,
-                      _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
-    "dli_scalar_gate_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr,
-                             _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int, _c_int,
-                             _c_float, _c_int, _c_ptr],
+                      _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr],
+    "dli_scalar_gate_scan": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr,
+                             _c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
+                             _c_int, _c_float, _c_int, _c_int, _c_ptr],
     "dli_group_norm": [_c_ptr, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_float, _c_int, _c_ptr],
     "dli_branch_norm_mean": [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_float, _c_ptr],
     "dli_head_norm_gate": [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_float, _c_ptr, _c_i64, _c_int, _c_int, _c_int, _c_int,
@@ -2230,13 +2230,13 @@ def head_products(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: Opt
 
 def exp_gates(pre: torch.Tensor, i_off: int, f_off: int, i_bias: Optional[torch.Tensor], f_bias: Optional[torch.Tensor],
               cap: float, state: torch.Tensor, m_off: int, q_start: torch.Tensor, positions: torch.Tensor,
-              state_slots: torch.Tensor, heads: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+              state_slots: torch.Tensor, heads: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """The factors of a matrix memory with exponential gates, per row and head of the step: from the float32
     pre-activations ``pre [n, >=]`` (input gate of head ``h`` at column ``i_off + h``, forget gate at
     ``f_off + h``; biases float32 ``[heads]``) the log gates ``i = cap tanh(. / cap)`` (``cap`` 0: as they are) and
     ``f = logsigmoid(cap tanh(. / cap))``, the running reference point ``m <- max(f + m, i)`` (kept at
     ``state[slot][m_off + h]``, 0 at position 0), and ``keep = exp(f + m_old - m)``, ``write = exp(i - m)``,
-    ``floor = exp(-m)``: three float32 ``[n, heads]``."""
+    ``floor = exp(-m)``, and the logarithm of ``keep`` (never above zero): four float32 ``[n, heads]``."""
     _f32_rows(pre, "pre")
     n = pre.shape[0]
     _require(0 <= i_off and i_off + heads <= pre.shape[1] and 0 <= f_off and f_off + heads <= pre.shape[1],
@@ -2247,25 +2247,29 @@ def exp_gates(pre: torch.Tensor, i_off: int, f_off: int, i_bias: Optional[torch.
             _require(t.shape[0] == heads, f"{name} must hold a value per head")
     _state_rows(state, m_off + heads)
     entries = _step_arrays(q_start, positions, state_slots, n)
-    out = torch.empty(3, n, heads, device=pre.device, dtype=torch.float32)
+    out = torch.empty(4, n, heads, device=pre.device, dtype=torch.float32)
     _check(library().dli_exp_gates(_ptr(pre), pre.stride(0), int(i_off), int(f_off), _ptr(i_bias), _ptr(f_bias), float(cap),
                                    _ptr(state), state.stride(0), int(m_off), _ptr(q_start), _ptr(positions), _ptr(state_slots),
-                                   _ptr(out[0]), _ptr(out[1]), _ptr(out[2]), entries, n, heads, _stream()), "exp_gates")
-    return out[0], out[1], out[2]
+                                   _ptr(out[0]), _ptr(out[1]), _ptr(out[2]), _ptr(out[3]), entries, n, heads, _stream()),
+           "exp_gates")
+    return out[0], out[1], out[2], out[3]
 
 
 def scalar_gate_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor,
                      positions: torch.Tensor, state_slots: torch.Tensor, o: torch.Tensor, heads: int, dim: int, vdim: int, *,
                      keep: Optional[torch.Tensor] = None, write: Optional[torch.Tensor] = None,
                      decay: Optional[torch.Tensor] = None, floor: Optional[torch.Tensor] = None,
-                     den: Optional[torch.Tensor] = None, q_scale: float = 1.0, silu: bool = False) -> None:
+                     den: Optional[torch.Tensor] = None, q_scale: float = 1.0, silu: bool = False,
+                     log_keep: Optional[torch.Tensor] = None, chunked: bool = True) -> None:
     """Per request and head ``S <- a S + b k v^T``, ``o = S^T q`` over the step's rows in order, with
     ``a, b = keep, write`` (float32 ``[n, heads]``) or ``a = decay[head]``, ``b = 1``. ``q, k [n, heads*dim]`` and
     ``v [n, heads*vdim]`` are float32 with contiguous rows (columns of a wider matrix will do); with ``silu`` all
     three pass through silu first; q is multiplied by ``q_scale``. With ``floor`` (float32 ``[n, heads]``) the state
     has one more column a head, for a value that is always one, and ``den [n, heads]`` receives
     ``max(|that column's result|, floor) + 1e-6``. ``S`` float32 ``[heads][vdim (+ 1)][dim]`` at the start of
-    ``state[slot]`` (zeros at position 0); ``o [n, heads*vdim]`` float32."""
+    ``state[slot]`` (zeros at position 0); ``o [n, heads*vdim]`` float32. A step with portions whose heads hold 16 to 64
+    keys in steps of 16 runs 64 tokens at a time on the matrix cores, in 32-bit (``chunked``; under gates it needs
+    ``log_keep``, the logarithm of ``keep``; not with ``silu``); any other walks the tokens one by one."""
     for name, t, width in (("q", q, heads * dim), ("k", k, heads * dim), ("v", v, heads * vdim), ("o", o, heads * vdim)):
         _f32_rows(t, name)
         _require(t.shape[1] == width, f"{name} must hold {width} columns")
@@ -2273,7 +2277,7 @@ def scalar_gate_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: t
     _require(k.shape[0] == n and v.shape[0] == n and o.shape[0] == n, "q, k, v and o differ in rows")
     _require((keep is None) == (write is None) and (keep is not None or decay is not None), "keep and write, or decay")
     _require((floor is None) == (den is None) and (floor is None or keep is not None), "floor and den come with the gates")
-    for name, t in (("keep", keep), ("write", write), ("floor", floor), ("den", den)):
+    for name, t in (("keep", keep), ("write", write), ("floor", floor), ("den", den), ("log_keep", log_keep)):
         if t is not None:
             _dense(t, name, torch.float32, 2)
             _require(t.shape == (n, heads), f"{name} must be [n, heads]")
@@ -2283,9 +2287,10 @@ def scalar_gate_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: t
     _state_rows(state, heads * (vdim + (floor is not None)) * dim)
     entries = _step_arrays(q_start, positions, state_slots, n)
     _check(library().dli_scalar_gate_scan(
-        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(keep), _ptr(write), heads, _ptr(decay),
-        _ptr(floor), _ptr(den), _ptr(state), state.stride(0), _ptr(q_start), _ptr(positions), _ptr(state_slots), _ptr(o),
-        o.stride(0), entries, n, heads, dim, vdim, float(q_scale), int(bool(silu)), _stream()), "scalar_gate_scan")
+        _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(keep), _ptr(write), _ptr(log_keep), heads,
+        _ptr(decay), _ptr(floor), _ptr(den), _ptr(state), state.stride(0), _ptr(q_start), _ptr(positions), _ptr(state_slots),
+        _ptr(o), o.stride(0), entries, n, heads, dim, vdim, float(q_scale), int(bool(silu)), int(bool(chunked)), _stream()),
+        "scalar_gate_scan")
 
 
 def diff_head_norm(a: torch.Tensor, lam: float, after: float, eps: float, gate: Optional[torch.Tensor], out: torch.Tensor,

@@ -374,13 +374,13 @@ class MatrixMemory(_ScalarGateMixer):
             proj = linear_f32(self.rt, as_operand(self.rt, x, ctx), self.w_in)
         k0, v0, g0 = self.hd, 2 * self.hd, 2 * self.hd + self.hv
         i0 = g0 + self.hv
-        keep, write, floor = ops.exp_gates(proj, i0, i0 + H, self.i_bias, self.f_bias, self.gate_cap, state, self.state_floats,
+        keep, write, floor, log_keep = ops.exp_gates(proj, i0, i0 + H, self.i_bias, self.f_bias, self.gate_cap, state, self.state_floats,
                                            ctx.q_start, ctx.positions, ctx.state_slots, H)
         o = torch.empty(n, self.hv, device=self.rt.device, dtype=torch.float32)
         den = torch.empty(n, H, device=self.rt.device, dtype=torch.float32)
         ops.scalar_gate_scan(proj[:, :k0], proj[:, k0:v0], proj[:, v0:g0], state, ctx.q_start, ctx.positions, ctx.state_slots,
                              o, H, self.head_dim, self.value_dim, keep=keep, write=write, floor=floor, den=den,
-                             q_scale=self.head_dim ** -0.5)
+                             log_keep=log_keep, q_scale=self.head_dim ** -0.5)
         out = self.rt.empty(n, self.hv)
         ops.head_norm_gate(o, proj[:, g0:g0 + self.hv], self.norm_w, self.norm_eps, out, H, self.value_dim, gate="sigmoid",
                            den=den)

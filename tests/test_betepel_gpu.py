@@ -177,9 +177,11 @@ def plain_memory(q, k, v, gi, gf, ib, fb, cap, dim):
     return P.matrix_memory(q * dim ** -0.5, k, v, i, P.log_sigmoid(f), {})
 
 
+@pytest.mark.parametrize("chunked", [True, False])
 @pytest.mark.parametrize("H,D,V,cap", [(2, 8, 6, 15.0), (4, 32, 48, 4.0), (1, 64, 16, 0.0), (3, 20, 70, 8.0), (2, 128, 3, 15.0),
-                                       (1, 16, 130, 2.0), (2, 48, 1, 30.0)])
-def test_matrix_memory_in_steps_against_whole(ops, H, D, V, cap):
+                                       (1, 16, 130, 2.0), (2, 48, 1, 30.0), (2, 64, 37, 15.0)])
+def test_matrix_memory_in_steps_against_whole(ops, H, D, V, cap, chunked):
+    """``chunked``: steps with portions run 64 tokens at a time on the matrix cores where the head's size allows."""
     g = torch.Generator().manual_seed(H * 100 + D)
     ib, fb = torch.randn(H, generator=g), torch.randn(H, generator=g) + 2.0
     width = 2 * H * D + H * V + 2 * H
@@ -190,11 +192,12 @@ def test_matrix_memory_in_steps_against_whole(ops, H, D, V, cap):
 
     def run(rows, q_start, positions, slots):
         n = rows.shape[0]
-        keep, write, floor = ops.exp_gates(rows, width - 2 * H, width - H, ib.cuda(), fb.cuda(), cap, state, floats, q_start,
-                                           positions, slots, H)
+        keep, write, floor, log_keep = ops.exp_gates(rows, width - 2 * H, width - H, ib.cuda(), fb.cuda(), cap, state, floats,
+                                                     q_start, positions, slots, H)
         o, den = torch.empty(n, H * V).cuda(), torch.empty(n, H).cuda()
         ops.scalar_gate_scan(rows[:, :H * D], rows[:, H * D:2 * H * D], rows[:, 2 * H * D:2 * H * D + H * V], state, q_start,
-                             positions, slots, o, H, D, V, keep=keep, write=write, floor=floor, den=den, q_scale=D ** -0.5)
+                             positions, slots, o, H, D, V, keep=keep, write=write, floor=floor, den=den, log_keep=log_keep,
+                             q_scale=D ** -0.5, chunked=chunked)
         return o.view(n, H, V) / den[:, :, None]
 
     got = in_steps(reqs, PLAN, run)
@@ -204,7 +207,8 @@ def test_matrix_memory_in_steps_against_whole(ops, H, D, V, cap):
         ref = plain_memory(x[:, :H * D].view(n, H, D), x[:, H * D:2 * H * D].view(n, H, D),
                            x[:, 2 * H * D:2 * H * D + H * V].view(n, H, V), x[:, width - 2 * H:width - H], x[:, width - H:],
                            ib.double(), fb.double(), cap, D)
-        assert (got[r].double() - ref).abs().max() < 3e-5 * max(1.0, ref.abs().max()), (r, (got[r].double() - ref).abs().max())
+        # (a denominator |n . q| is a sum that cancels: its last bits are worth 1e-4 of a result)
+        assert (got[r].double() - ref).abs().max() < 1e-4 * max(1.0, ref.abs().max()), (r, (got[r].double() - ref).abs().max())
     assert (state[:, floats + H:] == 55.0).all()
 
 
@@ -218,11 +222,11 @@ def test_the_reference_point_starts_at_zero_and_the_floor_holds_early(ops):
     rows = torch.cat([q, k, v, gi, gf], 1).cuda()
     state = torch.zeros(1, H * (V + 1) * D + H).cuda()
     qs, pos, sl = step_arrays([(0, 0, n)])
-    keep, write, floor = ops.exp_gates(rows, 2 * H * D + H * V, 2 * H * D + H * V + H, None, None, 0.0, state, H * (V + 1) * D, qs,
-                                       pos, sl, H)
+    keep, write, floor, log_keep = ops.exp_gates(rows, 2 * H * D + H * V, 2 * H * D + H * V + H, None, None, 0.0, state,
+                                                 H * (V + 1) * D, qs, pos, sl, H)
     o, den = torch.empty(n, H * V).cuda(), torch.empty(n, H).cuda()
     ops.scalar_gate_scan(rows[:, :D], rows[:, D:2 * D], rows[:, 2 * D:2 * D + V], state, qs, pos, sl, o, H, D, V, keep=keep,
-                         write=write, floor=floor, den=den, q_scale=D ** -0.5)
+                         write=write, floor=floor, den=den, log_keep=log_keep, q_scale=D ** -0.5)
     ref = plain_memory(q.double().view(n, H, D), k.double().view(n, H, D), v.double().view(n, H, V), gi.double(), gf.double(),
                        torch.zeros(H, dtype=F), torch.zeros(H, dtype=F), 0.0, D)
     got = (o.view(n, H, V) / den[:, :, None]).cpu().double()
@@ -230,8 +234,10 @@ def test_the_reference_point_starts_at_zero_and_the_floor_holds_early(ops):
     assert ref.abs().max() < 1e-2          # the floor, not the normaliser, decided
 
 
-@pytest.mark.parametrize("H,D,V", [(2, 8, 6), (3, 64, 32), (1, 16, 130), (2, 20, 7), (2, 96, 1)])
-def test_decayed_linear_attention_in_steps_against_whole(ops, H, D, V):
+@pytest.mark.parametrize("inside", [True, False])
+@pytest.mark.parametrize("H,D,V", [(2, 8, 6), (3, 64, 32), (1, 16, 130), (2, 20, 7), (2, 96, 1), (3, 48, 21)])
+def test_decayed_linear_attention_in_steps_against_whole(ops, H, D, V, inside):
+    """``inside``: silu inside the scan, token by token; else beforehand, and portions in chunks on the matrix cores."""
     g = torch.Generator().manual_seed(H * 10 + V)
     decay = torch.tensor([0.6, 0.97, 1.0][:H])
     reqs = {r: (SLOTS[r], torch.randn(n, 2 * H * D + H * V + 8, generator=g)) for r, n in LENGTHS.items()}
@@ -239,8 +245,11 @@ def test_decayed_linear_attention_in_steps_against_whole(ops, H, D, V):
 
     def run(rows, q_start, positions, slots):
         o = torch.empty(rows.shape[0], H * V).cuda()
+        if not inside:
+            rows = rows.clone()
+            ops.silu_columns(rows[:, 8:])
         ops.scalar_gate_scan(rows[:, 8:8 + H * D], rows[:, 8 + H * D:8 + 2 * H * D], rows[:, 8 + 2 * H * D:], state, q_start, positions,
-                             slots, o, H, D, V, decay=decay.cuda(), silu=True)
+                             slots, o, H, D, V, decay=decay.cuda(), silu=inside)
         return o
 
     got = in_steps(reqs, PLAN, run)
