@@ -301,21 +301,21 @@ def betepel_shape(width, heads, kv_heads, ff, layers, vocab, chunk):
     same window beside decayed linear attention with heads of 64; the matrix memory with heads of 64; every
     layer with the mixture of experts that every other Miberax layer has (32 experts of an eighth of the Llama
     layer's hidden size, four chosen, here by a table, beside a shared expert of a quarter)."""
-    rot = {"dims": 32, "base": 1e6, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}
-    diff = {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.5,
+    rot = {"dims": 32, "base": 5e5, "scaling": {"factor": 4.0, "low": 1.0, "high": 4.0, "original": 8192}}
+    diff = {"heads": heads // 2, "kv_heads": max(1, kv_heads // 2), "dim": 64, "vdim": 128, "scale": 0.125, "diff": 0.4,
             "mask": {"size": chunk, "keep_first": 64}, "rot": rot}
     pair = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": 64, "vdim": 64, "scale": 0.125, "mask": {"size": chunk},
                      "rot": {"dims": 64, "base": 1e6}},
             "right": {"heads": heads, "dim": 64, "vdim": 64, "decay": [1.0 - 2.0 ** -(3 + 5 * h / heads) for h in range(heads)]},
-            "left_scale": 0.8, "right_scale": 0.5}
-    memory = {"heads": heads, "dim": 64, "vdim": 64, "gate_cap": 15.0}
+            "left_scale": 0.7, "right_scale": 0.6}
+    memory = {"heads": heads, "dim": 64, "vdim": 64, "gate_cap": 10.0}
     mlp = {"kind": "moe", "expert": {"ff": ff // 8}, "router": {"experts": 32, "top": 4}, "shared": {"ff": ff // 4}}
     out = []
     for i in range(layers):
         kind = ("attention", "parallel", "mlstm", "attention")[i % 4]
         mixer = dict(diff, kv_from=i - 3) if i % 4 == 3 else {"attention": diff, "parallel": pair, "mlstm": memory}[kind]
         out.append({"type": kind, "mixer": mixer, "mlp": mlp})
-    return {"architecture": "Betepel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.25, "layers": out}
+    return {"architecture": "Betepel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "logit_scale": 0.5, "layers": out}
 
 
 DESIGN_SIZES = {  # width, heads (of 64), kv heads, feed-forward, layers, vocabulary, attention chunk

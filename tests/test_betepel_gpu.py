@@ -413,7 +413,7 @@ def _aligned():
     att = {"heads": 2, "kv_heads": 1, "dim": 16, "vdim": 32, "scale": 0.25, "diff": 0.6, "mask": {"size": 70, "keep_first": 66}, "rot": rot}
     left = {"heads": 4, "kv_heads": 2, "dim": 32, "vdim": 16, "scale": 0.18, "mask": {"size": 130}, "rot": {"dims": 16, "base": 5000.0}}
     right = {"heads": 2, "dim": 32, "vdim": 32, "decay": [0.9, 0.999]}
-    mem = {"heads": 2, "dim": 16, "vdim": 32, "gate_cap": 15.0}
+    mem = {"heads": 2, "dim": 16, "vdim": 32, "gate_cap": 12.0}
     m = moe(4, 1, 32, 64)
     return config(64, 90, 1.0, [layer("attention", att, m),
                                 layer("parallel", {"left": left, "right": right, "left_scale": 1.0, "right_scale": 0.25}, m),
