@@ -477,35 +477,38 @@ _REFS: dict = {}
 
 
 def reference(name, W, cfg, toks, dtype):
-    """The plain logits, and for bfloat16 also those of slightly jittered matrices: the distance between
-    the two, row by row, is what rounding of that size may do to the row."""
+    """The plain logits, and how far each row moves when the matrices are jittered by bfloat16's rounding (the larger of
+    two draws): what rounding of that size may do to the row. A difference of two attention maps, or a denominator
+    that is a sum which cancels, makes a row here and there a hundred times more sensitive than its neighbours."""
     key = (name, tuple(toks))
     if key not in _REFS:
-        _REFS[key] = (P.forward_logits(cfg, W, toks), P.forward_logits(cfg, P.jittered(W), toks))
-    ref, moved = _REFS[key]
-    return (ref, moved) if dtype == "bfloat16" else (ref, None)
+        ref = P.forward_logits(cfg, W, toks)
+        moved = [(P.forward_logits(cfg, P.jittered(W, seed=j), toks) - ref).abs().max(dim=-1, keepdim=True).values for j in (0, 5)]
+        _REFS[key] = (ref, torch.maximum(*moved))
+    return _REFS[key]
 
 
 def rows_of(ref, rows):
-    return tuple(None if r is None else r[rows] for r in ref)
+    return tuple(r[rows] for r in ref)
 
 
 def close(got: torch.Tensor, ref, dtype: str, what) -> None:
     """In 32-bit every row is held, and that is where a fault of the cache, the state, a window or the table
-    shows (it moves rows by 1e-2 and more). In bfloat16 a row may be off by bfloat16's usual share of its
-    largest logit and a few times what a jitter of that size on the matrices does to it."""
+    shows (it moves rows by 1e-2 and more); a row that a jitter of bfloat16's size moves by a tenth of its largest
+    logit may be off by a thousandth of that. In bfloat16 a row may be off by bfloat16's usual share of its
+    largest logit and a few times what such a jitter does to it."""
     ref, moved = ref
     got, ref = got.double().cpu(), ref.double()
     assert got.shape == ref.shape, what
     err = (got - ref).abs()
     top = ref.abs().max(dim=-1, keepdim=True).values.clamp(min=1.0)
-    if moved is not None:
-        slack = 8 * (moved.double() - ref).abs().max(dim=-1, keepdim=True).values
-        bad = (err > 8e-2 * top + slack).any(dim=-1)
+    if dtype == "bfloat16":
+        bad = (err > 8e-2 * top + 8 * moved).any(dim=-1)
         assert not bad.any(), (what, bad.nonzero().flatten().tolist())
         assert (err / top).max(dim=-1).values.median() < 4e-2, (what, (err / top).max(dim=-1).values.median())
         return
-    assert (err / top).max() < 2e-4, (what, (err / top).max())
+    assert (err <= 2e-4 * top + 1e-3 * moved).all(), (what, (err / top).max())
+    assert (err / top).max(dim=-1).values.median() < 2e-5, (what, (err / top).max(dim=-1).values.median())
 
 
 def prompt(cfg, n, seed):
@@ -648,6 +651,106 @@ def test_mixed_batches_with_pages_and_slots_used_again(name, dtype, page_size, t
     for i in reqs:
         assert at[i] == len(reqs[i])
         close(torch.cat(got[i]), refs[i], dtype, (name, i))
+
+
+def drawn_config(seed: int) -> dict:
+    """A model whose sizes, order of layers, windows and constants are drawn from ``seed``."""
+    rng = random.Random(seed)
+    width, vocab = rng.choice([96, 128, 160, 192, 256]), rng.randrange(150, 700)
+
+    def rotation(dim):
+        if rng.random() < 0.15:
+            return None
+        rot = {"dims": rng.choice([d for d in (2, 4, 8, 12, 16, 24, 32, 48, 64) if d <= dim]), "base": rng.choice([100.0, 1e4, 5e5])}
+        if rng.random() < 0.5:
+            rot["scaling"] = {"factor": rng.choice([2.0, 8.0]), "low": 1.0, "high": rng.choice([2.0, 4.0]), "original": rng.choice([32, 64, 256])}
+        return rot
+
+    def heads_pair():
+        kv = rng.choice([1, 2, 3])
+        return kv * rng.choice([1, 2, 3]), kv
+
+    def mlp():
+        if rng.random() < 0.15:
+            return None
+        experts = rng.randrange(1, 9)
+        return moe(experts, rng.randrange(1, min(experts, 3) + 1), rng.choice([16, 24, 32, 64]), rng.choice([None, 32, 48]))
+
+    layers, lenders = [], []
+    for i in range(rng.randrange(3, 7)):
+        kind = rng.choice(["attention", "attention", "parallel", "mlstm"])
+        if kind == "attention":
+            if lenders and rng.random() < 0.5:
+                mixer = dict(layers[rng.choice(lenders)]["mixer"], kv_from=None)
+                mixer["kv_from"] = layers.index(next(l for l in layers if l["mixer"] is not mixer and l["type"] == "attention"
+                                                        and l["mixer"].get("kv_from") is None and l["mixer"]["heads"] == mixer["heads"]
+                                                        and l["mixer"]["dim"] == mixer["dim"] and l["mixer"]["vdim"] == mixer["vdim"]
+                                                        and l["mixer"]["kv_heads"] == mixer["kv_heads"] and l["mixer"].get("rot") == mixer.get("rot")))
+            else:
+                h, kv = heads_pair()
+                dim = rng.choice([16, 24, 32, 48, 64])
+                mixer = {"heads": h, "kv_heads": kv, "dim": dim, "vdim": rng.choice([16, 32, 40, 64, 96]), "scale": dim ** -0.5 * rng.choice([1.0, 1.5]),
+                         "diff": rng.choice([0.2, 0.5, 0.7]), "rot": rotation(dim)}
+                if mixer["rot"] is None:
+                    del mixer["rot"]
+                lenders.append(i)
+            mixer["mask"] = {"size": rng.randrange(5, 120), "keep_first": rng.choice([0, 1, 7, 20, 70])}
+            if rng.random() < 0.1:
+                del mixer["mask"]
+        elif kind == "parallel":
+            h, kv = heads_pair()
+            dim = rng.choice([16, 32, 48, 64])
+            left = {"heads": h, "kv_heads": kv, "dim": dim, "vdim": rng.choice([16, 32, 48]), "scale": dim ** -0.5, "mask": {"size": rng.randrange(5, 150)},
+                    "rot": rotation(dim)}
+            if left["rot"] is None:
+                del left["rot"]
+            rh = rng.randrange(1, 5)
+            right = {"heads": rh, "dim": rng.choice([16, 24, 32, 64]), "vdim": rng.choice([8, 16, 32, 40]),
+                     "decay": [rng.choice([0.6, 0.9, 0.97, 0.999, 1.0]) for _ in range(rh)]}
+            mixer = {"left": left, "right": right, "left_scale": rng.choice([0.5, 1.0]), "right_scale": rng.choice([0.3, 1.2])}
+        else:
+            mixer = {"heads": rng.randrange(1, 5), "dim": rng.choice([16, 24, 32, 64]), "vdim": rng.choice([16, 32, 40, 64]),
+                     "gate_cap": rng.choice([5.0, 15.0, 30.0])}
+        layers.append(layer(kind, mixer, mlp()))
+        layers[-1]["mixer"] = mixer          # (the same dictionary, so that a borrower finds its lender)
+    return config(width, vocab, rng.choice([0.25, 1.0, 2.0]), layers, eps=rng.choice([1e-5, 1e-6]))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(8))
+def test_models_of_drawn_sizes_whole_in_portions_decoded_and_mixed(seed, dtype, tmp_root):
+    """Sizes, order of layers, windows, kept positions, rotations, tables and constants drawn at random: whole prompts, portions
+    that change in size, a decoded tail, and two requests beside each other, each against the plain model."""
+    name = f"drawn{seed}"
+    if name not in _MODELS:
+        cfg = drawn_config(seed)
+        W = P.random_weights(cfg, seed=100 + seed)
+        _MODELS[name] = (cfg, W, P.write_folder(tmp_root / name, cfg, W))
+    cfg, W, folder = _MODELS[name]
+    a, b = prompt(cfg, 170, 40 + seed), prompt(cfg, 61, 60 + seed)
+    ra, rb = reference(name, W, cfg, a, dtype), reference(name, W, cfg, b, dtype)
+    s = session(folder, dtype, pages=24, graphs=dtype == "bfloat16")
+    close(s.step([{"id": "w", "tokens": a, "want": list(range(len(a)))}], end=["w"]), ra, dtype, (name, "whole"))
+    rows, at = {"a": [], "b": []}, {"a": 0, "b": 0}
+    toks = {"a": a, "b": b}
+    plan = [[("a", 37)], [("a", 2), ("b", 30)], [("b", 1), ("a", 64)], [("a", 3), ("b", 1)], [("a", 40), ("b", 2)], [("b", 27)]]
+    plan += [[("a", 1)]] * 24
+    for step in plan:
+        entries, end = [], []
+        for r, n in step:
+            entries.append({"id": r, "tokens": toks[r][at[r]:at[r] + n], "want": list(range(n))})
+            at[r] += n
+            if at[r] == len(toks[r]):
+                end.append(r)
+        out = s.step(entries, end=end)
+        r0 = 0
+        for r, n in step:
+            rows[r].append(out[r0:r0 + n])
+            r0 += n
+    assert at == {"a": len(a), "b": len(b)}
+    close(torch.cat(rows["a"]), ra, dtype, (name, "a"))
+    close(torch.cat(rows["b"]), rb, dtype, (name, "b"))
+    s.core.manager.check_invariants()
 
 
 def test_a_row_does_not_depend_on_its_batch(tmp_root):
